@@ -1,0 +1,402 @@
+/*
+ * dt_oracle.c -- CPU restatement of the FP8 / MX quantization path of driss_torch.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  It is the checker the HIP kernels are
+ * compared against; only tests, the smoke check and the benchmark's cpu_baseline leg may
+ * load it.  Nothing shipped routes through it.
+ *
+ * Every routine is scalar, bit-level C (no library float8 types) so that it is independent
+ * of the PyTorch conversions it is pinned against in tests/test_oracle_*.py.
+ *
+ * Reference citations (paths relative to the reference tree):
+ *   amax                     test/test_amax.py:6-7            abs().max() as fp32
+ *   scale                    test/test_sat_cast.py:35         tensor_to_scale (torchao, absent from
+ *                            the reference tree, unpinned version): f32(fmax / max(f64(amax), 1e-12))
+ *   saturated cast           test/test_sat_cast.py:7-24       a*scale, where-clamp to +-fmax, .to(fp8)
+ *                            src/saturated_cast.cu:59-104     bf16 product rounded to bf16 (mode V2)
+ *   dynamic_scaled_quant     test/test_dynamic_quant.py:36-44, src/dynamic_scaled_quant.cu:83-118
+ *   MX exponent / E8M0 byte  src/mx_cast.cu:44-86,146-155
+ *   blocked scale layout     test/test_mx.py:28-32 (transformer_nuggets to_blocked, absent from the
+ *                            reference tree, unpinned), length check src/mx_fp8_bf16.cu:197-205
+ *   MX GEMM                  test/test_mx.py:34-39, src/mx_fp8_bf16.cu:217-241
+ *
+ * Pinning (see tests/): fp8/bf16 converts are checked exhaustively against torch's CPU
+ * `.to(float8_*)` over all 2^16 bf16 patterns and a dense fp32 sweep, and against the
+ * known-answer vectors in tests/golden/; amax/scale/cast against the eager formulation;
+ * the MX exponent against ceil(log2) in exact (float64 / integer) arithmetic; to_blocked
+ * against the view/permute formulation; the GEMM against brute force and float64 matmul.
+ * Documented choices where the third-party oracle (torchao) is version dependent and no
+ * vector in the reference pins it ("parity unpinned" corners): a block holding a NaN gets
+ * scale byte 255 and an all-NaN payload; scale byte 0 decodes to 2^-127 (its E8M0 value);
+ * subnormal fp32 block maxima use exponent -126 as src/mx_cast.cu:57-59 does.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+
+#define DTO_EXPORT __attribute__((visibility("default")))
+
+/* dtype codes shared with include/driss_torch_hip.h */
+enum { DTO_F32 = 0, DTO_BF16 = 1, DTO_F16 = 2 };
+enum { DTO_E4M3FN = 0, DTO_E5M2 = 1 };
+/* product rounding modes of x*scale for bf16 input (fp32 input: all three coincide) */
+enum { DTO_ROUND_V1 = 1, /* bf16(f32(x) * s)            : eager, 0-dim CPU scale            */
+       DTO_ROUND_V2 = 2, /* bf16(f32(x) * f32(bf16(s))) : reference kernel, 0-dim GPU scale */
+       DTO_ROUND_V3 = 3  /* f32(x) * s                  : eager, scale of rank >= 1         */ };
+
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+DTO_EXPORT float dto_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+/* round-to-nearest-even fp32 -> bf16; NaN is kept a (quiet) NaN */
+DTO_EXPORT uint16_t dto_f32_to_bf16(float f) {
+  uint32_t u = f2u(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+DTO_EXPORT float dto_f16_to_f32(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t e = (h >> 10) & 0x1Fu, m = h & 0x3FFu;
+  if (e == 0) {
+    if (m == 0) return u2f(sign);
+    float v = (float)m * 0x1p-24f; /* subnormal: m * 2^-24 */
+    return u2f(f2u(v) | sign);
+  }
+  if (e == 31) return u2f(sign | 0x7F800000u | (m << 13));
+  return u2f(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+/*
+ * Generic IEEE-style fp32 -> small float, round to nearest even, NO saturation: this is
+ * what `.to(torch.float8_*)` does and therefore what follows the explicit clamp of
+ * test/test_sat_cast.py:19-24.  ebits/mbits describe the target, `fn` selects the
+ * "finite only" e4m3fn encoding (no inf, single NaN mantissa pattern).
+ */
+static uint8_t f32_to_fp8_generic(float f, int ebits, int mbits, int fn) {
+  uint32_t u = f2u(f);
+  uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+  uint32_t a = u & 0x7FFFFFFFu;
+  const int bias = (1 << (ebits - 1)) - 1;
+  const uint8_t nan_code = 0x7F; /* e4m3fn: S.1111.111 ; e5m2: S.11111.11 */
+  const uint8_t inf_code = (uint8_t)(((1u << ebits) - 1u) << mbits); /* e5m2 only */
+  if (a > 0x7F800000u) return sign | nan_code;
+  if (a == 0x7F800000u) return sign | (fn ? nan_code : inf_code);
+  if (a == 0) return sign;
+  int e = (int)(a >> 23) - 127; /* unbiased, fp32 subnormals treated below */
+  uint32_t m = a & 0x7FFFFFu;
+  if ((a >> 23) == 0) { /* fp32 subnormal: far below any fp8 subnormal -> rounds to 0 */
+    return sign;
+  }
+  m |= 0x800000u; /* 24-bit significand, value = m * 2^(e-23) */
+  /* target quantum exponent: normal -> e - mbits ; subnormal -> (1-bias) - mbits */
+  int emin = 1 - bias;
+  int q = (e < emin ? emin : e) - mbits; /* result = round(m * 2^(e-23-q)) * 2^q */
+  int shift = (e - 23) - q;              /* <= 0 always: we drop -shift bits */
+  int drop = -shift;
+  uint32_t r;
+  if (drop >= 32) {
+    r = 0;
+  } else {
+    uint32_t keep = m >> drop;
+    uint32_t rem = m & ((1u << drop) - 1u);
+    uint32_t half = 1u << (drop - 1);
+    if (rem > half || (rem == half && (keep & 1u))) keep++;
+    r = keep;
+  }
+  /* r is the significand in units of 2^q; renormalise (it may have carried) */
+  if (r == 0) return sign;
+  int rexp; /* biased target exponent */
+  uint32_t rm;
+  if (r < (1u << mbits)) { /* subnormal */
+    rexp = 0;
+    rm = r;
+  } else {
+    int eq = q + mbits; /* unbiased exponent if r in [2^mbits, 2^(mbits+1)) */
+    while (r >= (2u << mbits)) { r >>= 1; eq++; } /* exact: only happens as 2^(mbits+1) */
+    rexp = eq + bias;
+    rm = r & ((1u << mbits) - 1u);
+  }
+  uint32_t code = ((uint32_t)rexp << mbits) | rm;
+  if (fn) {
+    if (code >= 0x7Fu) return sign | nan_code; /* beyond 448 -> NaN (no inf in e4m3fn) */
+  } else {
+    if (rexp >= (1 << ebits) - 1) return sign | inf_code; /* overflow -> inf */
+  }
+  return sign | (uint8_t)code;
+}
+
+DTO_EXPORT uint8_t dto_f32_to_e4m3fn(float f) { return f32_to_fp8_generic(f, 4, 3, 1); }
+DTO_EXPORT uint8_t dto_f32_to_e5m2(float f) { return f32_to_fp8_generic(f, 5, 2, 0); }
+
+DTO_EXPORT float dto_e4m3fn_to_f32(uint8_t b) {
+  uint32_t s = (uint32_t)(b & 0x80u) << 24;
+  uint32_t e = (b >> 3) & 0xFu, m = b & 7u;
+  if (e == 15 && m == 7) return u2f(s | 0x7FC00000u);
+  if (e == 0) return u2f(f2u((float)m * 0x1p-9f) | s);
+  return u2f(s | ((e + 120u) << 23) | (m << 20));
+}
+
+DTO_EXPORT float dto_e5m2_to_f32(uint8_t b) {
+  uint32_t s = (uint32_t)(b & 0x80u) << 24;
+  uint32_t e = (b >> 2) & 0x1Fu, m = b & 3u;
+  if (e == 31) return u2f(s | 0x7F800000u | (m ? 0x400000u : 0u));
+  if (e == 0) return u2f(f2u((float)m * 0x1p-16f) | s);
+  return u2f(s | ((e + 112u) << 23) | (m << 21));
+}
+
+/* E8M0 decode: 2^(b-127); 255 is NaN.  b == 0 is 2^-127 (an fp32 subnormal). */
+DTO_EXPORT float dto_e8m0_to_f32(uint8_t b) {
+  if (b == 255) return u2f(0x7FC00000u);
+  if (b == 0) return u2f(0x00400000u);
+  return u2f((uint32_t)b << 23);
+}
+
+static inline float fp8_max_of(int out_dtype) { return out_dtype == DTO_E5M2 ? 57344.0f : 448.0f; }
+
+static inline float load_as_f32(const void* x, int in_dtype, size_t i) {
+  switch (in_dtype) {
+    case DTO_F32: return ((const float*)x)[i];
+    case DTO_BF16: return dto_bf16_to_f32(((const uint16_t*)x)[i]);
+    default: return dto_f16_to_f32(((const uint16_t*)x)[i]);
+  }
+}
+
+/* ---------------------------------------------------------------- amax ------------- */
+/* test/test_amax.py:6-7: torch.abs(a).max().to(float32).  NaN propagates (torch.max does). */
+DTO_EXPORT float dto_amax(const void* x, int in_dtype, int64_t numel) {
+  float best = 0.0f;
+  int seen_nan = 0;
+  for (int64_t i = 0; i < numel; ++i) {
+    float v = fabsf(load_as_f32(x, in_dtype, (size_t)i));
+    if (v != v) seen_nan = 1;
+    else if (v > best) best = v;
+  }
+  return seen_nan ? u2f(0x7FC00000u) : best;
+}
+
+/* per-row amax: amax(dim=-1, keepdim=True) of the eager rowwise formulation */
+DTO_EXPORT void dto_amax_rows(const void* x, int in_dtype, int64_t rows, int64_t cols, float* out) {
+  size_t esz = in_dtype == DTO_F32 ? 4 : 2;
+  for (int64_t r = 0; r < rows; ++r)
+    out[r] = dto_amax((const char*)x + (size_t)r * (size_t)cols * esz, in_dtype, cols);
+}
+
+/* torchao amax_to_scale as used through tensor_to_scale (test/test_sat_cast.py:35):
+ * res = fmax / clamp(amax.to(float64), min=1e-12); res.to(float32) */
+DTO_EXPORT float dto_amax_to_scale(float amax, int out_dtype) {
+  double a = (double)amax;
+  double c = a != a ? a : (a < 1e-12 ? 1e-12 : a); /* clamp keeps NaN */
+  return (float)((double)fp8_max_of(out_dtype) / c);
+}
+
+/* ------------------------------------------------------ saturated cast -------------- */
+/* one element of eager_scaled_quant (test/test_sat_cast.py:7-24) under a product
+ * rounding mode; the two torch.where clamps leave NaN untouched. */
+DTO_EXPORT uint8_t dto_scaled_quant_one(float x, int x_is_bf16, float scale, int out_dtype, int mode) {
+  float p;
+  if (x_is_bf16 && mode == DTO_ROUND_V2) {
+    float sb = dto_bf16_to_f32(dto_f32_to_bf16(scale));
+    p = dto_bf16_to_f32(dto_f32_to_bf16(x * sb));
+  } else if (x_is_bf16 && mode == DTO_ROUND_V1) {
+    p = dto_bf16_to_f32(dto_f32_to_bf16(x * scale));
+  } else {
+    p = x * scale;
+  }
+  const float fmax = fp8_max_of(out_dtype);
+  if (p > fmax) p = fmax;
+  if (p < -fmax) p = -fmax;
+  return out_dtype == DTO_E5M2 ? dto_f32_to_e5m2(p) : dto_f32_to_e4m3fn(p);
+}
+
+DTO_EXPORT void dto_saturated_cast(const void* x, int in_dtype, int64_t numel, float scale,
+                                   int out_dtype, int mode, uint8_t* out) {
+  const int is_bf16 = in_dtype == DTO_BF16;
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < numel; ++i)
+    out[i] = dto_scaled_quant_one(load_as_f32(x, in_dtype, (size_t)i), is_bf16, scale, out_dtype, mode);
+}
+
+/* per-tensor dynamic quant: amax -> scale -> cast (test/test_dynamic_quant.py:36-44) */
+DTO_EXPORT void dto_dynamic_scaled_quant(const void* x, int in_dtype, int64_t numel, int out_dtype,
+                                         int mode, uint8_t* out, float* amax_out, float* scale_out) {
+  float a = dto_amax(x, in_dtype, numel);
+  float s = dto_amax_to_scale(a, out_dtype);
+  if (amax_out) *amax_out = a;
+  if (scale_out) *scale_out = s;
+  dto_saturated_cast(x, in_dtype, numel, s, out_dtype, mode, out);
+}
+
+/* rowwise dynamic quant: scale has shape [rows,1] so eager promotes to fp32 (mode V3) */
+DTO_EXPORT void dto_dynamic_scaled_quant_rowwise(const void* x, int in_dtype, int64_t rows, int64_t cols,
+                                                 int out_dtype, uint8_t* out, float* amax_out,
+                                                 float* scale_out) {
+  size_t esz = in_dtype == DTO_F32 ? 4 : 2;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    const char* row = (const char*)x + (size_t)r * (size_t)cols * esz;
+    float a = dto_amax(row, in_dtype, cols);
+    float s = dto_amax_to_scale(a, out_dtype);
+    if (amax_out) amax_out[r] = a;
+    if (scale_out) scale_out[r] = s;
+    for (int64_t c = 0; c < cols; ++c)
+      out[r * cols + c] = dto_scaled_quant_one(load_as_f32(row, in_dtype, (size_t)c), 0, s, out_dtype,
+                                               DTO_ROUND_V3);
+  }
+}
+
+/* ----------------------------------------------------------- MX cast ---------------- */
+/* src/mx_cast.cu:50-65: ceil(log2|x|) from the fp32 exponent field */
+DTO_EXPORT int dto_mx_ceil_log2(float absval) {
+  uint32_t bits = f2u(absval) & 0x7FFFFFFFu;
+  int be = (int)(bits >> 23);
+  if (be == 0) return bits == 0 ? -128 : -126;
+  return be - 127 + ((bits & 0x7FFFFFu) ? 1 : 0);
+}
+
+/* src/mx_cast.cu:71-79: biased E8M0 byte = clamp(max_log2 - target_pow2 + 127, 0, 255);
+ * target_pow2 is 8 for e4m3 (the reference hard-codes it) and 15 for e5m2. */
+DTO_EXPORT uint8_t dto_mx_scale_byte(int max_log2, int out_dtype) {
+  int b = max_log2 - (out_dtype == DTO_E5M2 ? 15 : 8) + 127;
+  if (b < 0) b = 0;
+  if (b > 254) b = 254; /* 255 is reserved for NaN; unreachable for finite input */
+  return (uint8_t)b;
+}
+
+/* quantize one block of `n` strided elements; returns the scale byte */
+static uint8_t mx_block(const void* x, int in_dtype, size_t first, size_t stride, int n, int out_dtype,
+                        uint8_t* data, size_t dfirst, size_t dstride) {
+  int mx = -128, has_nan = 0;
+  for (int i = 0; i < n; ++i) {
+    float v = load_as_f32(x, in_dtype, first + (size_t)i * stride);
+    if (v != v) has_nan = 1;
+    int l = dto_mx_ceil_log2(fabsf(v));
+    if (l > mx) mx = l;
+  }
+  const float fmax = fp8_max_of(out_dtype);
+  if (has_nan) {
+    for (int i = 0; i < n; ++i) data[dfirst + (size_t)i * dstride] = 0x7F;
+    return 255;
+  }
+  uint8_t sb = dto_mx_scale_byte(mx, out_dtype);
+  int k = 127 - (int)sb; /* payload = x * 2^k, exact */
+  for (int i = 0; i < n; ++i) {
+    float v = load_as_f32(x, in_dtype, first + (size_t)i * stride);
+    float p = (float)ldexp((double)v, k); /* exact scaling, then one rounding to fp32 */
+    if (p > fmax) p = fmax;
+    if (p < -fmax) p = -fmax;
+    data[dfirst + (size_t)i * dstride] = out_dtype == DTO_E5M2 ? dto_f32_to_e5m2(p) : dto_f32_to_e4m3fn(p);
+  }
+  return sb;
+}
+
+/*
+ * MX quantization of a row-major [rows, cols] matrix with 32-element blocks.
+ *  axis = 1: blocks run along a row (src/mx_cast.cu:96-161); cols % 32 == 0.
+ *            data [rows, cols], scale [rows, cols/32] row-major.
+ *  axis = 0: blocks run down a column; rows % 32 == 0.
+ *            transpose = 0: data [rows, cols], scale [rows/32, cols]
+ *            transpose = 1: data [cols, rows], scale [cols, rows/32]  (== axis-1 cast of x^T)
+ *  axis = 1 with transpose = 1: data [cols, rows], scale [cols/32, rows].
+ */
+DTO_EXPORT int dto_mx_quantize(const void* x, int in_dtype, int64_t rows, int64_t cols, int axis,
+                               int transpose, int out_dtype, uint8_t* data, uint8_t* scale) {
+  if (axis == 1) {
+    if (cols % 32) return -1;
+    int64_t nb = cols / 32;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r)
+      for (int64_t b = 0; b < nb; ++b) {
+        size_t first = (size_t)(r * cols + b * 32);
+        uint8_t s;
+        if (!transpose) {
+          s = mx_block(x, in_dtype, first, 1, 32, out_dtype, data, first, 1);
+          scale[r * nb + b] = s;
+        } else {
+          s = mx_block(x, in_dtype, first, 1, 32, out_dtype, data, (size_t)(b * 32 * rows + r), (size_t)rows);
+          scale[b * rows + r] = s;
+        }
+      }
+  } else {
+    if (rows % 32) return -1;
+    int64_t nb = rows / 32;
+#pragma omp parallel for schedule(static)
+    for (int64_t b = 0; b < nb; ++b)
+      for (int64_t c = 0; c < cols; ++c) {
+        size_t first = (size_t)(b * 32 * cols + c);
+        uint8_t s;
+        if (!transpose) {
+          s = mx_block(x, in_dtype, first, (size_t)cols, 32, out_dtype, data, first, (size_t)cols);
+          scale[b * cols + c] = s;
+        } else {
+          s = mx_block(x, in_dtype, first, (size_t)cols, 32, out_dtype, data, (size_t)(c * rows + b * 32), 1);
+          scale[c * nb + b] = s;
+        }
+      }
+  }
+  return 0;
+}
+
+/* ----------------------------------------------- blocked 128x4 scale layout --------- */
+/* byte offset of scale (r, c) of an [R, C] scale matrix in the cuBLAS block-scaling layout
+ * that mx_fp8_bf16 consumes (test/test_mx.py:31-32; size check src/mx_fp8_bf16.cu:197-205) */
+DTO_EXPORT int64_t dto_blocked_offset(int64_t r, int64_t c, int64_t C) {
+  int64_t cb = (C + 3) / 4;
+  return ((r / 128) * cb + c / 4) * 512 + (r % 32) * 16 + ((r % 128) / 32) * 4 + (c % 4);
+}
+
+DTO_EXPORT int64_t dto_blocked_size(int64_t R, int64_t C) { return 128 * ((R + 127) / 128) * 4 * ((C + 3) / 4); }
+
+DTO_EXPORT void dto_to_blocked(const uint8_t* scale, int64_t R, int64_t C, uint8_t* out) {
+  memset(out, 0, (size_t)dto_blocked_size(R, C));
+  for (int64_t r = 0; r < R; ++r)
+    for (int64_t c = 0; c < C; ++c) out[dto_blocked_offset(r, c, C)] = scale[r * C + c];
+}
+
+/* ------------------------------------------------------------ MX GEMM --------------- */
+/*
+ * D[M,N] = sum_k (A[m,k] * 2^(sfa[m,k/32]-127)) * (B[n,k] * 2^(sfb[n,k/32]-127))
+ * a: e4m3 [M,K] row-major (lda bytes between rows); bt: e4m3 [N,K] row-major, i.e. the
+ * reference's `b` of shape [K,N] with stride(0)==1 (src/mx_fp8_bf16.cu:208-213);
+ * sfa/sfb in the blocked layout.  Accumulates in float64 (the exact value is what a
+ * "dequantized fp32 matmul" approximates) and writes fp32.  O(MNK): small sizes only.
+ */
+DTO_EXPORT void dto_mx_gemm_ref(const uint8_t* a, const uint8_t* bt, const uint8_t* sfa,
+                                const uint8_t* sfb, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                int64_t ldb, float* out) {
+  int64_t KB = (K + 31) / 32;
+  float lut[256];
+  for (int i = 0; i < 256; ++i) lut[i] = dto_e4m3fn_to_f32((uint8_t)i);
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m)
+    for (int64_t n = 0; n < N; ++n) {
+      double acc = 0.0;
+      for (int64_t kb = 0; kb < KB; ++kb) {
+        double part = 0.0;
+        int64_t k1 = (kb + 1) * 32 < K ? (kb + 1) * 32 : K;
+        for (int64_t k = kb * 32; k < k1; ++k) part += (double)lut[a[m * lda + k]] * (double)lut[bt[n * ldb + k]];
+        int ea = (int)sfa[dto_blocked_offset(m, kb, KB)] - 127;
+        int eb = (int)sfb[dto_blocked_offset(n, kb, KB)] - 127;
+        acc += ldexp(part, ea + eb);
+      }
+      out[m * N + n] = (float)acc;
+    }
+}
+
+/* dequantize an MX operand to fp32: out[r,c] = e4m3(data[r,c]) * 2^(scale-127), plain
+ * [R, C/32] scale layout (what mx_fp8_quantize emits) */
+DTO_EXPORT void dto_mx_dequant(const uint8_t* data, const uint8_t* scale, int64_t R, int64_t C,
+                               int out_dtype, float* out) {
+  int64_t nb = C / 32;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < R; ++r)
+    for (int64_t c = 0; c < C; ++c) {
+      uint8_t b = data[r * C + c];
+      float v = out_dtype == DTO_E5M2 ? dto_e5m2_to_f32(b) : dto_e4m3fn_to_f32(b);
+      uint8_t s = scale[r * nb + c / 32];
+      out[r * C + c] = s == 255 ? u2f(0x7FC00000u) : (float)ldexp((double)v, (int)s - 127);
+    }
+}

@@ -1,0 +1,148 @@
+"""Pins the MX part of the oracle: exponent formula against exact ceil(log2) arithmetic,
+C oracle against the eager restatement, the blocked layout against its view/permute
+definition, the GEMM reference against float64 matmul and brute force."""
+import ctypes as C
+import json
+import math
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from oracle import eager
+
+GOLD = Path(__file__).parent / "golden"
+
+
+def _student_t(shape, seed, df=3.0):
+    g = torch.Generator().manual_seed(seed)
+    n = torch.randn(shape, generator=g)
+    chi = sum(torch.randn(shape, generator=g) ** 2 for _ in range(int(df)))
+    return n / torch.sqrt(chi / df)
+
+
+def test_mx_exponent_matches_exact_ceil_log2():
+    lib = co.lib()
+    g = torch.Generator().manual_seed(1)
+    vals = torch.cat([torch.rand(5000, generator=g) * 1000, torch.linspace(-30, 30, 61).exp2(), torch.tensor([16.125, 0.999, 448.0])]).float()
+    for v in vals.tolist():
+        # exact: frexp gives v = m * 2^e with m in [0.5, 1): ceil(log2 v) = e-1 if m == 0.5 else e
+        m, e = math.frexp(v)
+        exact = e - 1 if m == 0.5 else e
+        assert lib.dto_mx_ceil_log2(C.c_float(v)) == exact
+    assert lib.dto_mx_ceil_log2(C.c_float(0.0)) == -128  # src/mx_cast.cu:59
+    assert lib.dto_mx_ceil_log2(C.c_float(1e-40)) == -126  # subnormal, src/mx_cast.cu:59
+    ev = eager.mx_ceil_exponent(vals)
+    assert ev.tolist() == [lib.dto_mx_ceil_log2(C.c_float(v)) for v in vals.tolist()]
+
+
+def test_mx_golden_scale_bytes():
+    kat = json.loads((GOLD / "mx_kat.json").read_text())
+    for row in kat["scale_byte"]:
+        v = np.array([int(row["max_abs_bits"], 16)], dtype=np.uint32).view(np.float32)[0]
+        x = torch.zeros(1, 32, dtype=torch.float32)
+        x[0, 7] = -float(v)
+        x[0, 8] = float(v) / 3
+        data, scale = co.mx_quantize(x)
+        assert int(scale[0, 0]) == row["e4m3_scale_byte"], row
+        # dequantized max element is within one e4m3 ulp (2^-3 relative) of the input
+        deq = co.mx_dequant(data, scale)
+        if v > 0:
+            assert abs(deq[0, 7].item() + v) <= v * 2**-3
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("out_dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+def test_mx_c_oracle_vs_eager(in_dtype, out_dtype):
+    a = _student_t((64, 256), 21).to(in_dtype)
+    a[3, 32:64] = 0  # all-zero block -> byte 0, zero payload
+    a[5, 70] = 3e4 if in_dtype != torch.float16 else 6e4
+    data, scale = co.mx_quantize(a, out_dtype=out_dtype)
+    rs, rd = eager.to_mx(a, out_dtype)
+    assert torch.equal(scale, rs)
+    assert torch.equal(data, rd.view(torch.uint8))
+    assert scale[3, 1] == 0 and (data[3, 32:64] == 0).all()
+
+
+def test_mx_block_properties():
+    """per block: the scaled max lies in (2^7, 2^8], so after rounding to e4m3 the payload max
+    magnitude lies in [2^7, 2^8]; dequantization error <= 2^-4 * blockmax (e4m3 has 3 mantissa bits, scaled
+    max <= 256 -> quantum 32 at the top binade) -- catches an off-by-one in the exponent."""
+    a = _student_t((128, 512), 22).to(torch.bfloat16)
+    data, scale = co.mx_quantize(a)
+    deq = co.mx_dequant(data, scale)
+    x = a.float().reshape(128, 16, 32)
+    bm = x.abs().amax(-1)
+    pm = data.view(torch.float8_e4m3fn).float().reshape(128, 16, 32).abs().amax(-1)
+    assert ((pm >= 128) & (pm <= 256)).all()
+    err = (deq.reshape(128, 16, 32) - x).abs().amax(-1)
+    assert (err <= bm * 2**-4).all()
+
+
+@pytest.mark.parametrize("transpose", [False, True])
+def test_mx_axis0_is_axis1_of_transpose(transpose):
+    a = _student_t((96, 64), 23).to(torch.bfloat16)
+    d0, s0 = co.mx_quantize(a, axis=0, transpose=transpose)
+    dT, sT = co.mx_quantize(a.T.contiguous(), axis=1)
+    if transpose:
+        assert torch.equal(d0, dT) and torch.equal(s0, sT)
+    else:
+        assert torch.equal(d0, dT.T) and torch.equal(s0, sT.T)
+    d1t, s1t = co.mx_quantize(a, axis=1, transpose=True)
+    d1, s1 = co.mx_quantize(a, axis=1)
+    assert torch.equal(d1t, d1.T) and torch.equal(s1t, s1.T)
+
+
+@pytest.mark.parametrize("shape", [(128, 4), (256, 8), (129, 5), (133, 16), (1, 1), (640, 64)])
+def test_to_blocked_matches_view_permute_definition(shape):
+    g = torch.Generator().manual_seed(31)
+    s = torch.randint(1, 255, shape, generator=g, dtype=torch.int32).to(torch.uint8)
+    ref = eager.to_blocked(s)
+    got = co.to_blocked(s)
+    assert torch.equal(ref, got)
+    R, Cc = shape
+    # length = 128*ceil(R/128)*4*ceil(C/4); equals the operator's check when C % 4 == 0
+    assert got.numel() == 128 * ((R + 127) // 128) * 4 * ((Cc + 3) // 4)
+    lib = co.lib()
+    for r, c in [(0, 0), (R - 1, Cc - 1), (R // 2, Cc // 2)]:
+        assert int(got[lib.dto_blocked_offset(r, c, Cc)]) == int(s[r, c])
+
+
+def _mx_operands(M, N, K, seed):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    b = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    ad, asc = co.mx_quantize(a)
+    bd, bsc = co.mx_quantize(b)
+    return ad, asc, bd, bsc
+
+
+@pytest.mark.parametrize("size", [(32, 16, 64), (129, 40, 128), (64, 64, 256)])
+def test_mx_gemm_reference(size):
+    M, N, K = size
+    ad, asc, bd, bsc = _mx_operands(M, N, K, 41)
+    got = co.mx_gemm_ref(ad, bd, co.to_blocked(asc), co.to_blocked(bsc))
+    ref64 = (co.mx_dequant(ad, asc).double() @ co.mx_dequant(bd, bsc).double().T)
+    torch.testing.assert_close(got.double(), ref64, rtol=1e-6, atol=1e-6)
+    ref_eager = eager.mx_gemm_ref(ad.view(torch.float8_e4m3fn), asc, bd.view(torch.float8_e4m3fn), bsc)
+    assert eager.compute_error(ref64, ref_eager) > 120
+    # brute force one entry with python floats
+    m, n = M // 2, N // 3
+    da, db = co.mx_dequant(ad, asc), co.mx_dequant(bd, bsc)
+    acc = sum(float(da[m, k]) * float(db[n, k]) for k in range(K))
+    assert abs(acc - float(got[m, n])) <= 1e-5 * max(1.0, abs(acc))
+
+
+def test_mx_gemm_scale_linearity():
+    """bumping one operand's scale bytes by +1 doubles the matching contribution: a property
+    that fails if scales are applied to the wrong rows / k-blocks."""
+    M, N, K = 32, 32, 128
+    ad, asc, bd, bsc = _mx_operands(M, N, K, 43)
+    base = co.mx_gemm_ref(ad, bd, co.to_blocked(asc), co.to_blocked(bsc))
+    asc2 = asc.clone()
+    asc2[7, :] += 1
+    out = co.mx_gemm_ref(ad, bd, co.to_blocked(asc2), co.to_blocked(bsc))
+    torch.testing.assert_close(out[7], base[7] * 2)
+    assert torch.equal(out[:7], base[:7]) and torch.equal(out[8:], base[8:])
