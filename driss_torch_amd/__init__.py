@@ -1,0 +1,116 @@
+"""driss_torch on MI355X: FP8 / MX quantization ops behind ``torch.ops.DrissTorch``.
+
+The wrapper names, signatures and defaults follow the reference's
+``driss_torch/__init__.py:20-122``; the work is done by hand-written gfx950 kernels in
+``lib/libdriss_torch_hip.so`` (C ABI: ``include/driss_torch_hip.h``) reached through the
+registration shim ``lib/libdriss_torch.so``.  There is no fallback path: importing this
+package fails if the libraries have not been built (``python -m driss_torch_amd._build``).
+"""
+from pathlib import Path
+from typing import Optional, Tuple
+
+import torch
+
+_LIB_DIR = Path(__file__).parent / "lib"
+hip_lib_path = _LIB_DIR / "libdriss_torch_hip.so"
+lib_path = _LIB_DIR / "libdriss_torch.so"
+for _p in (hip_lib_path, lib_path):
+    if not _p.exists():
+        raise ImportError(f"{_p} is missing: build it with `python -m driss_torch_amd._build`")
+torch.ops.load_library(str(lib_path.resolve()))
+torch.ops.import_module("driss_torch_amd.abstract_impls")
+
+ops = torch.ops.DrissTorch
+Tensor = torch.Tensor
+
+# product rounding of x*scale for bf16 inputs (see include/driss_torch_hip.h: dt_round_mode)
+ROUND_AUTO, ROUND_BF16_PRODUCT, ROUND_BF16_SCALE_PRODUCT, ROUND_F32 = 0, 1, 2, 3
+
+
+def saturated_cast(x: Tensor, scale: Tensor, out_dtype: torch.dtype, transpose: bool = False) -> Tensor:
+    """fp8 saturated cast of ``x * scale`` (reference: driss_torch/__init__.py:20-38).
+
+    ``scale`` is a one-element fp32 tensor on the device.  For bf16 ``x`` the product is
+    rounded the way eager PyTorch rounds it for that scale tensor: a 0-dim scale keeps the
+    product (and the scale) in bf16, a scale of rank >= 1 promotes the product to fp32.
+    """
+    assert not transpose, "Transpose is not supported yet"
+    return ops.saturated_cast(x, scale, out_dtype, transpose)
+
+
+def saturated_cast_mode(x: Tensor, scale: Tensor, out_dtype: torch.dtype, mode: int) -> Tensor:
+    """``saturated_cast`` with the product rounding mode given explicitly (ROUND_*)."""
+    return ops.saturated_cast_mode(x, scale, out_dtype, False, mode)
+
+
+def amax(x: Tensor) -> Tensor:
+    """max(abs(x)) as an fp32 tensor of shape [1] (reference: driss_torch/__init__.py:41-43)."""
+    return ops.amax(x)
+
+
+def dynamic_scaled_quant(inpt: Tensor, dtype: torch.dtype) -> Tensor:
+    """amax -> scale -> saturated cast in one call (reference: driss_torch/__init__.py:46-47)."""
+    return ops.dynamic_scaled_quant(inpt, dtype)
+
+
+def dynamic_scaled_quant_ex(inpt: Tensor, dtype: torch.dtype, mode: int = ROUND_AUTO) -> Tuple[Tensor, Tensor, Tensor]:
+    """As ``dynamic_scaled_quant`` but also returns (amax [1], scale 0-dim)."""
+    return ops.dynamic_scaled_quant_ex(inpt, dtype, mode)
+
+
+def dynamic_scaled_quant_pair(inpt: Tensor, mode: int = ROUND_AUTO) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """e4m3fn and e5m2 casts from one amax and one read: (e4m3fn, e5m2, amax [1], scale [2])."""
+    return ops.dynamic_scaled_quant_pair(inpt, mode)
+
+
+def dynamic_scaled_quant_rowwise(inpt: Tensor, dtype: torch.dtype) -> Tuple[Tensor, Tensor, Tensor]:
+    """Per-row scales: (fp8 [R,C], amax [R,1], scale [R,1]); the product is taken in fp32."""
+    return ops.dynamic_scaled_quant_rowwise(inpt, dtype)
+
+
+def sweep_mm(x: Tensor, w: Tensor, x_scale: Tensor, w_scale: Tensor, bias: Optional[Tensor], out_dtype: torch.dtype,
+             use_fast_accum: bool, cluster_shape_x: int, cluster_shape_y: int, cluster_shape_z: int, transposed: bool,
+             swizzle: int) -> Tensor:
+    """Schema kept from the reference (driss_torch/__init__.py:50-77); not built, raises."""
+    return ops.sweep_mm(x, w, x_scale, w_scale, bias, out_dtype, use_fast_accum, cluster_shape_x, cluster_shape_y,
+                        cluster_shape_z, transposed, swizzle)
+
+
+def mx_fp8_bf16(a: Tensor, b: Tensor, a_scale: Tensor, b_scale: Tensor) -> Tensor:
+    """bf16 = (a * 2^a_scale) @ (b * 2^b_scale) for e4m3fn operands with E8M0 block-32 scales
+    in the blocked 128x4 layout (reference: driss_torch/__init__.py:80-94).
+
+    a: [M, K] row-major; b: [K, N] with stride(0) == 1 (an [N, K] tensor transposed).
+    """
+    return ops.mx_fp8_bf16(a, b, a_scale, b_scale)
+
+
+def mx_fp4_bf16(a: Tensor, b: Tensor, a_scale: Tensor, b_scale: Tensor) -> Tensor:
+    """Schema kept from the reference (driss_torch/__init__.py:97-111); not built, raises."""
+    return ops.mx_fp4_bf16(a, b, a_scale, b_scale)
+
+
+def mx_fp8_quantize(input: Tensor, block_size: int = 32, axis: int = 1, transpose: bool = False,
+                    ScalarType: torch.dtype = torch.float8_e4m3fn) -> Tuple[Tensor, Tensor]:
+    """MXFP8 cast (reference: driss_torch/__init__.py:114-122): (payload, E8M0 scales, 1-D).
+
+    axis 1 blocks along rows, axis 0 down columns.  Payload is [M, N], or [N, M] with
+    ``transpose``; the flat scale tensor is the row-major scale matrix [M, N/32] (axis 1),
+    [M/32, N] (axis 0), [N/32, M] (axis 1, transpose) or [N, M/32] (axis 0, transpose).
+    """
+    return ops.mx_fp8_quantize(input, block_size, axis, transpose, ScalarType)
+
+
+mx_cast = mx_fp8_quantize
+
+
+def mx_fp8_quantize_blocked(input: Tensor, axis: int = 1, ScalarType: torch.dtype = torch.float8_e4m3fn
+                            ) -> Tuple[Tensor, Tensor]:
+    """MXFP8 cast whose scales come out in the blocked layout ``mx_fp8_bf16`` reads, with K as
+    the contiguous payload dimension: axis 1 -> payload [M, N]; axis 0 -> payload [N, M]."""
+    return ops.mx_fp8_quantize_ex(input, 32, axis, axis % 2 == 0, ScalarType, True)
+
+
+def to_blocked(scale: Tensor) -> Tensor:
+    """[R, C] E8M0 scale matrix -> flat blocked 128x4 layout (zero padded)."""
+    return ops.to_blocked(scale)

@@ -1,0 +1,108 @@
+// Status strings, device facts, tuning knobs and the workspace entry points of the C ABI.
+#include <string.h>
+
+#include <mutex>
+
+#include "dt_device.hpp"
+#include "dt_host.hpp"
+
+namespace dt {
+
+namespace {
+struct Knob {
+  const char* key;
+  int value;
+};
+// Launch-shape knobs.  Workgroups per CU for the persistent grids, chosen on MI355X.
+Knob g_knobs[] = {
+    {"amax.blocks_per_cu", 8},
+    {"cast.blocks_per_cu", 8},
+    {"cast.nontemporal", 0},
+    {"dynamic.cooperative", 0},
+    {"mx.blocks_per_cu", 8},
+    {"mx.col_rbw", 0},
+    {"gemm.variant", 0},
+};
+constexpr int kNumKnobs = sizeof(g_knobs) / sizeof(g_knobs[0]);
+
+constexpr int kMaxDevices = 16;
+DeviceFacts g_facts[kMaxDevices];
+std::once_flag g_facts_once[kMaxDevices];
+}  // namespace
+
+int tuning(const char* key) {
+  for (int i = 0; i < kNumKnobs; ++i)
+    if (strcmp(g_knobs[i].key, key) == 0) return g_knobs[i].value;
+  return 0;
+}
+
+const DeviceFacts& device_facts() {
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  if (dev < 0 || dev >= kMaxDevices) dev = 0;
+  std::call_once(g_facts_once[dev], [dev] {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    g_facts[dev].cu_count = cus;
+  });
+  return g_facts[dev];
+}
+
+__global__ void zero_words_kernel(uint32_t* p, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+}  // namespace dt
+
+extern "C" {
+
+const char* dt_status_string(int status) {
+  switch (status) {
+    case DT_OK: return "ok";
+    case DT_ERR_INVALID_DTYPE: return "unsupported dtype";
+    case DT_ERR_INVALID_SHAPE: return "invalid shape";
+    case DT_ERR_NULL_POINTER: return "null pointer";
+    case DT_ERR_MISALIGNED: return "misaligned pointer";
+    case DT_ERR_WORKSPACE: return "workspace missing or too small";
+    case DT_ERR_INVALID_MODE: return "invalid mode";
+    case DT_ERR_LAUNCH: return "kernel launch failed";
+    case DT_ERR_EMPTY: return "reduction over zero elements";
+    default: return "unknown status";
+  }
+}
+
+int dt_abi_version(void) { return 1; }
+
+size_t dt_workspace_bytes(void) { return dt::kWsBytes; }
+
+int dt_workspace_init(void* workspace, size_t workspace_bytes, dt_stream_t stream) {
+  if (!workspace) return DT_ERR_NULL_POINTER;
+  if (workspace_bytes < dt::kWsBytes) return DT_ERR_WORKSPACE;
+  if (!dt::aligned(workspace, 256)) return DT_ERR_MISALIGNED;
+  // a fill kernel rather than hipMemsetAsync, so the call is safe under graph capture
+  dt::zero_words_kernel<<<1, 64, 0, dt::as_hip(stream)>>>(static_cast<uint32_t*>(workspace), 64);
+  return dt::launch_status();
+}
+
+int dt_set_tuning(const char* key, int value) {
+  if (!key) return DT_ERR_NULL_POINTER;
+  for (int i = 0; i < dt::kNumKnobs; ++i)
+    if (strcmp(dt::g_knobs[i].key, key) == 0) {
+      dt::g_knobs[i].value = value;
+      return DT_OK;
+    }
+  return DT_ERR_INVALID_MODE;
+}
+
+int dt_get_tuning(const char* key, int* value) {
+  if (!key || !value) return DT_ERR_NULL_POINTER;
+  for (int i = 0; i < dt::kNumKnobs; ++i)
+    if (strcmp(dt::g_knobs[i].key, key) == 0) {
+      *value = dt::g_knobs[i].value;
+      return DT_OK;
+    }
+  return DT_ERR_INVALID_MODE;
+}
+
+}  // extern "C"

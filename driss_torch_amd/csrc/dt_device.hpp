@@ -1,0 +1,155 @@
+// Device-side building blocks shared by the gfx950 kernels: 16-byte vector access, bf16/f16
+// unpacking, OCP fp8 packing with the hardware converts, wave64 reductions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "driss_torch_hip.h"
+
+namespace dt {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float as_f32(uint32_t u) { return __uint_as_float(u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __float_as_uint(f); }
+
+// ------------------------------------------------------------------ element unpacking
+// A 32-bit word holds two bf16 / f16 values; lo = element with the lower address.
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return as_f32(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return as_f32(w & 0xFFFF0000u); }
+__device__ __forceinline__ float f16_lo(uint32_t w) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xFFFFu));
+}
+__device__ __forceinline__ float f16_hi(uint32_t w) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+}
+
+// fp32 -> bf16 -> fp32, round to nearest even, NaN stays NaN.
+__device__ __forceinline__ float round_to_bf16(float f) {
+  uint32_t u = as_u32(f);
+  uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
+  return (f != f) ? as_f32(u | 0x00400000u) : as_f32(r);
+}
+
+// ------------------------------------------------------------------------ fp8 packing
+template <int OUT>
+__device__ __forceinline__ constexpr float fp8_max() {
+  return OUT == DT_E5M2 ? 57344.0f : 448.0f;
+}
+
+// clamp to +-fmax with one v_med3_f32.  A NaN input does not survive med3, so callers that
+// must keep NaN patch the converted byte afterwards (see pack2 below).
+template <int OUT>
+__device__ __forceinline__ float clamp_fp8(float p) {
+  return __builtin_amdgcn_fmed3f(p, -fp8_max<OUT>(), fp8_max<OUT>());
+}
+
+// Two floats -> two fp8 bytes in the low (HI=false) or high (HI=true) half of `old`, using
+// v_cvt_pk_fp8_f32 / v_cvt_pk_bf8_f32 (round to nearest even, OCP encodings on gfx950).
+template <int OUT, bool HI>
+__device__ __forceinline__ uint32_t cvt_pk(float a, float b, uint32_t old) {
+  if constexpr (OUT == DT_E5M2)
+    return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(a, b, (int)old, HI);
+  else
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, HI);
+}
+
+// Saturating convert of four products to four packed fp8 bytes (byte i = p_i).  NaN inputs
+// become the canonical fp8 NaN with the input's sign (0x7F / 0xFF), which is what
+// `.to(torch.float8_*)` produces after the where-clamps leave a NaN in place.
+template <int OUT>
+__device__ __forceinline__ uint32_t pack4(float p0, float p1, float p2, float p3) {
+  uint32_t w = cvt_pk<OUT, false>(clamp_fp8<OUT>(p0), clamp_fp8<OUT>(p1), 0u);
+  w = cvt_pk<OUT, true>(clamp_fp8<OUT>(p2), clamp_fp8<OUT>(p3), w);
+  const bool any_nan = (p0 != p0) | (p1 != p1) | (p2 != p2) | (p3 != p3);
+  if (__builtin_expect(any_nan, 0)) {
+    auto fix = [&](float p, int sh) {
+      if (p != p) w = (w & ~(0xFFu << sh)) | ((0x7Fu | ((as_u32(p) >> 24) & 0x80u)) << sh);
+    };
+    fix(p0, 0); fix(p1, 8); fix(p2, 16); fix(p3, 24);
+  }
+  return w;
+}
+
+// Product x*scale under the three rounding modes of dt_round_mode.  `sb` is the scale
+// already rounded for the mode (bf16-rounded for mode 2), so modes 1 and 2 share code.
+template <bool ROUND_PRODUCT_TO_BF16>
+__device__ __forceinline__ float scaled(float x, float s) {
+  float p = x * s;
+  if constexpr (ROUND_PRODUCT_TO_BF16) p = round_to_bf16(p);
+  return p;
+}
+
+// -------------------------------------------------------------------- wave reductions
+// DPP cross-lane moves.  bound_ctrl=true makes invalid source lanes read 0, which is the
+// identity for an unsigned max.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+constexpr int kDppQuadXor1 = 0xB1;      // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;      // quad_perm:[2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141;
+constexpr int kDppRowMirror = 0x140;
+
+__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
+
+// max over the 4 lanes of a quad, result in all 4 lanes
+__device__ __forceinline__ uint32_t quad_umax(uint32_t v) {
+  v = umax(v, dpp<kDppQuadXor1>(v));
+  v = umax(v, dpp<kDppQuadXor2>(v));
+  return v;
+}
+
+// max over all 64 lanes, result in every lane: 4 DPP steps inside a row of 16, then two
+// ds_swizzle/bpermute exchanges across rows.
+__device__ __forceinline__ uint32_t wave_umax(uint32_t v) {
+  v = quad_umax(v);
+  v = umax(v, dpp<kDppRowHalfMirror>(v));
+  v = umax(v, dpp<kDppRowMirror>(v));
+  v = umax(v, (uint32_t)__shfl_xor((int)v, 16, kWave));
+  v = umax(v, (uint32_t)__shfl_xor((int)v, 32, kWave));
+  return v;
+}
+
+// max over a workgroup of NWAVES waves through LDS; result valid in every thread.
+template <int NWAVES>
+__device__ __forceinline__ uint32_t block_umax(uint32_t v, uint32_t* lds /* >= NWAVES words */) {
+  v = wave_umax(v);
+  if constexpr (NWAVES == 1) return v;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  if (lane == 0) lds[wave] = v;
+  __syncthreads();
+  uint32_t r = lds[0];
+#pragma unroll
+  for (int i = 1; i < NWAVES; ++i) r = umax(r, lds[i]);
+  __syncthreads();
+  return r;
+}
+
+// ------------------------------------------------------------------- magnitudes as ints
+// |x| of IEEE floats orders like its bit pattern read as an unsigned integer, and every
+// NaN pattern sorts above infinity, so an integer max both finds the amax and propagates NaN.
+__device__ __forceinline__ uint32_t absbits_f32(uint32_t w) { return w & 0x7FFFFFFFu; }
+
+// max |.| of the two bf16/f16 halves of a word, as a 16-bit pattern in each half (v_pk_max_u16)
+__device__ __forceinline__ uint32_t pk_absmax16(uint32_t acc, uint32_t w) {
+  u16x2 a = __builtin_bit_cast(u16x2, acc);
+  u16x2 b = __builtin_bit_cast(u16x2, w & 0x7FFF7FFFu);
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
+}
+
+// amax -> scale exactly as f32(fmax / max(f64(amax), 1e-12)); NaN propagates.
+__device__ __forceinline__ float amax_to_scale(float amax, float fmax) {
+  double a = (double)amax;
+  double c = (a != a) ? a : (a < 1e-12 ? 1e-12 : a);
+  return (float)((double)fmax / c);
+}
+
+}  // namespace dt

@@ -1,0 +1,72 @@
+// dt_dynamic_scaled_quant*: amax -> scale -> saturating fp8 cast, per tensor and per row (C ABI).
+//
+// Per tensor the work is two stream-ordered kernels: the amax reduction, whose last
+// workgroup also derives the scale(s) into the workspace, and the streaming cast, which
+// reads the scale from there.  The second read of x is served from the memory-side cache
+// for tensors that fit it.
+#include "quant_kernels.hpp"
+#include "rowwise_kernels.hpp"
+
+namespace {
+inline float fmax_of(int out_dtype) { return out_dtype == DT_E5M2 ? 57344.0f : 448.0f; }
+}  // namespace
+
+extern "C" int dt_dynamic_scaled_quant(const void* x, int in_dtype, int64_t numel, int out_dtype, int round_mode,
+                                       void* out, float* amax_out, float* scale_out, void* workspace,
+                                       size_t workspace_bytes, dt_stream_t stream) {
+  if (int st = dt::check_cast_args(x, in_dtype, numel, out_dtype, round_mode, out)) return st;
+  if (numel == 0) return DT_ERR_EMPTY;
+  if (int st = dt::check_workspace(workspace, workspace_bytes)) return st;
+  hipStream_t s = dt::as_hip(stream);
+  const float fm = fmax_of(out_dtype);
+  int st = in_dtype == DT_F32 ? dt::launch_amax<DT_F32>(x, numel, workspace, amax_out, scale_out, 1, fm, 0.f, s)
+                              : dt::launch_amax<DT_BF16>(x, numel, workspace, amax_out, scale_out, 1, fm, 0.f, s);
+  if (st) return st;
+  const float* scale = reinterpret_cast<const float*>(static_cast<const uint8_t*>(workspace) + dt::kWsScale);
+  return dt::launch_cast<false>(x, in_dtype, numel, scale, out_dtype, round_mode, out, nullptr, s);
+}
+
+extern "C" int dt_amax_scales(const void* x, int in_dtype, int64_t numel, float* amax_out, float* scale_out,
+                              void* workspace, size_t workspace_bytes, dt_stream_t stream) {
+  if (in_dtype != DT_F32 && in_dtype != DT_BF16) return DT_ERR_INVALID_DTYPE;
+  if (numel < 0) return DT_ERR_INVALID_SHAPE;
+  if (numel == 0) return DT_ERR_EMPTY;
+  if (!x) return DT_ERR_NULL_POINTER;
+  if (!dt::aligned(x, in_dtype == DT_F32 ? 4 : 2)) return DT_ERR_MISALIGNED;
+  if (int st = dt::check_workspace(workspace, workspace_bytes)) return st;
+  hipStream_t s = dt::as_hip(stream);
+  return in_dtype == DT_F32 ? dt::launch_amax<DT_F32>(x, numel, workspace, amax_out, scale_out, 2, 448.0f, 57344.0f, s)
+                            : dt::launch_amax<DT_BF16>(x, numel, workspace, amax_out, scale_out, 2, 448.0f, 57344.0f, s);
+}
+
+extern "C" int dt_saturated_cast_pair(const void* x, int in_dtype, int64_t numel, const float* scale, int round_mode,
+                                      void* out_e4m3fn, void* out_e5m2, dt_stream_t stream) {
+  if (int st = dt::check_cast_args(x, in_dtype, numel, DT_E4M3FN, round_mode, out_e4m3fn)) return st;
+  if (numel > 0 && !out_e5m2) return DT_ERR_NULL_POINTER;
+  if (!scale) return DT_ERR_NULL_POINTER;
+  if (!dt::aligned(scale, 4)) return DT_ERR_MISALIGNED;
+  if (numel == 0) return DT_OK;
+  return dt::launch_cast<true>(x, in_dtype, numel, scale, DT_E4M3FN, round_mode, out_e4m3fn, out_e5m2, dt::as_hip(stream));
+}
+
+extern "C" int dt_dynamic_scaled_quant_pair(const void* x, int in_dtype, int64_t numel, int round_mode,
+                                            void* out_e4m3fn, void* out_e5m2, float* amax_out, float* scale_out,
+                                            void* workspace, size_t workspace_bytes, dt_stream_t stream) {
+  if (int st = dt::check_cast_args(x, in_dtype, numel, DT_E4M3FN, round_mode, out_e4m3fn)) return st;
+  if (!out_e5m2) return DT_ERR_NULL_POINTER;
+  if (int st = dt_amax_scales(x, in_dtype, numel, amax_out, scale_out, workspace, workspace_bytes, stream)) return st;
+  const float* scale = reinterpret_cast<const float*>(static_cast<const uint8_t*>(workspace) + dt::kWsScale);
+  return dt_saturated_cast_pair(x, in_dtype, numel, scale, round_mode, out_e4m3fn, out_e5m2, stream);
+}
+
+extern "C" int dt_dynamic_scaled_quant_rowwise(const void* x, int in_dtype, int64_t rows, int64_t cols, int out_dtype,
+                                               void* out, float* amax_out, float* scale_out, dt_stream_t stream) {
+  if (in_dtype != DT_F32 && in_dtype != DT_BF16) return DT_ERR_INVALID_DTYPE;
+  if (out_dtype != DT_E4M3FN && out_dtype != DT_E5M2) return DT_ERR_INVALID_DTYPE;
+  if (rows < 0 || cols < 0) return DT_ERR_INVALID_SHAPE;
+  if (rows == 0) return DT_OK;
+  if (cols == 0) return DT_ERR_EMPTY;
+  if (!x || !out) return DT_ERR_NULL_POINTER;
+  if (!dt::aligned(x, in_dtype == DT_F32 ? 4 : 2)) return DT_ERR_MISALIGNED;
+  return dt::launch_rowwise(x, in_dtype, rows, cols, out_dtype, out, amax_out, scale_out, dt::as_hip(stream));
+}

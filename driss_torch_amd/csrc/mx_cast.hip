@@ -1,0 +1,130 @@
+// dt_mx_fp8_quantize / dt_to_blocked: MXFP8 cast with E8M0 block-32 scales (C ABI).
+#include "mx_kernels.hpp"
+
+namespace {
+using namespace dt;
+
+struct MxArgs {
+  const void* x;
+  int64_t rows, cols;
+  int axis, transpose;
+  uint8_t* data;
+  uint8_t* scale;
+  hipStream_t stream;
+};
+
+template <int IN, int OUT, int LAYOUT>
+int launch_mx(const MxArgs& a) {
+  constexpr int kV = InTraits<IN>::kVec;
+  const int64_t numel = a.rows * a.cols, nblocks = numel / 32;
+  const int cus = device_facts().cu_count;
+  const bool x_vec = aligned(a.x, 16);
+  if (a.axis == 1 && !a.transpose && x_vec && aligned(a.data, 8) && nblocks < (1ll << 28)) {
+    const int64_t nsuper = ceil_div(nblocks, 64);
+    int64_t waves = (int64_t)cus * tuning("mx.blocks_per_cu") * (kBlock / kWave);
+    if (waves > nsuper) waves = nsuper;
+    const unsigned grid = (unsigned)ceil_div(waves, kBlock / kWave);
+    mx_row_kernel<IN, OUT, LAYOUT><<<grid, kBlock, 0, a.stream>>>(a.x, (uint32_t)nblocks, (uint32_t)(a.cols / 32),
+                                                                 a.data, a.scale);
+    return launch_status();
+  }
+  if (a.axis == 0 && x_vec && a.cols % kV == 0 && aligned(a.data, 16) && aligned(a.scale, 8) &&
+      a.rows < (1ll << 31) && a.cols < (1ll << 31) && (LAYOUT == DT_SCALE_PLAIN || a.transpose)) {
+    const int64_t row_tiles = a.rows / 32, col_tiles = ceil_div(a.cols, (int64_t)kWave * kV);
+    auto waves_for = [&](int rbw) { return ceil_div(row_tiles, rbw) * col_tiles; };
+    int rbw = 1;
+    if (a.transpose) {
+      const int64_t enough = (int64_t)cus * 8;
+      int knob = tuning("mx.col_rbw");
+      rbw = knob ? knob : (waves_for(4) >= enough ? 4 : waves_for(2) >= enough ? 2 : 1);
+    }
+    const unsigned grid = (unsigned)ceil_div(waves_for(rbw), kBlock / kWave);
+    const uint32_t R = (uint32_t)a.rows, C = (uint32_t)a.cols;
+    if (!a.transpose) {
+      if constexpr (LAYOUT == DT_SCALE_PLAIN)
+        mx_col_kernel<IN, OUT, false, DT_SCALE_PLAIN, 1><<<grid, kBlock, 0, a.stream>>>(a.x, R, C, a.data, a.scale);
+    } else if (rbw == 4) {
+      mx_col_kernel<IN, OUT, true, LAYOUT, 4><<<grid, kBlock, 0, a.stream>>>(a.x, R, C, a.data, a.scale);
+    } else if (rbw == 2) {
+      mx_col_kernel<IN, OUT, true, LAYOUT, 2><<<grid, kBlock, 0, a.stream>>>(a.x, R, C, a.data, a.scale);
+    } else {
+      mx_col_kernel<IN, OUT, true, LAYOUT, 1><<<grid, kBlock, 0, a.stream>>>(a.x, R, C, a.data, a.scale);
+    }
+    return launch_status();
+  }
+  // general orientation / alignment
+  int64_t outer, inner_blocks, xos, xes, dos, des, s_rows, s_cols;
+  int s_t;
+  if (a.axis == 1) {
+    outer = a.rows; inner_blocks = a.cols / 32; xos = a.cols; xes = 1;
+    if (!a.transpose) { dos = a.cols; des = 1; s_rows = a.rows; s_cols = inner_blocks; s_t = 0; }
+    else { dos = 1; des = a.rows; s_rows = inner_blocks; s_cols = a.rows; s_t = 1; }
+  } else {
+    outer = a.cols; inner_blocks = a.rows / 32; xos = 1; xes = a.cols;
+    if (!a.transpose) { dos = 1; des = a.cols; s_rows = inner_blocks; s_cols = a.cols; s_t = 1; }
+    else { dos = a.rows; des = 1; s_rows = a.cols; s_cols = inner_blocks; s_t = 0; }
+  }
+  const int64_t total = outer * inner_blocks;
+  if (ceil_div(total, kBlock) > 0x7FFFFFFFll) return DT_ERR_INVALID_SHAPE;
+  mx_any_kernel<IN, OUT, LAYOUT><<<(unsigned)ceil_div(total, kBlock), kBlock, 0, a.stream>>>(
+      a.x, outer, inner_blocks, xos, xes, dos, des, s_rows, s_cols, s_t, a.data, a.scale);
+  return launch_status();
+}
+
+template <int IN>
+int launch_mx_in(const MxArgs& a, int out_dtype, int layout) {
+  if (out_dtype == DT_E4M3FN)
+    return layout == DT_SCALE_BLOCKED ? launch_mx<IN, DT_E4M3FN, DT_SCALE_BLOCKED>(a) : launch_mx<IN, DT_E4M3FN, DT_SCALE_PLAIN>(a);
+  return layout == DT_SCALE_BLOCKED ? launch_mx<IN, DT_E5M2, DT_SCALE_BLOCKED>(a) : launch_mx<IN, DT_E5M2, DT_SCALE_PLAIN>(a);
+}
+}  // namespace
+
+extern "C" int64_t dt_blocked_scale_bytes(int64_t R, int64_t C) {
+  if (R < 0 || C < 0) return 0;
+  return 128 * dt::ceil_div(R, 128) * 4 * dt::ceil_div(C, 4);
+}
+
+extern "C" int dt_mx_fp8_quantize(const void* x, int in_dtype, int64_t rows, int64_t cols, int axis, int transpose,
+                                  int out_dtype, int scale_layout, void* data, uint8_t* scale, dt_stream_t stream) {
+  if (in_dtype != DT_F32 && in_dtype != DT_BF16 && in_dtype != DT_F16) return DT_ERR_INVALID_DTYPE;
+  if (out_dtype != DT_E4M3FN && out_dtype != DT_E5M2) return DT_ERR_INVALID_DTYPE;
+  if ((axis != 0 && axis != 1) || (transpose != 0 && transpose != 1)) return DT_ERR_INVALID_MODE;
+  if (scale_layout != DT_SCALE_PLAIN && scale_layout != DT_SCALE_BLOCKED) return DT_ERR_INVALID_MODE;
+  if (rows < 0 || cols < 0) return DT_ERR_INVALID_SHAPE;
+  if ((axis == 1 ? cols : rows) % 32 != 0) return DT_ERR_INVALID_SHAPE;
+  // the blocked layout is defined for a scale matrix [outer, inner/32]
+  if (scale_layout == DT_SCALE_BLOCKED && !((axis == 1 && !transpose) || (axis == 0 && transpose))) return DT_ERR_INVALID_MODE;
+  if (rows == 0 || cols == 0) return DT_OK;
+  if (!x || !data || !scale) return DT_ERR_NULL_POINTER;
+  if (!dt::aligned(x, in_dtype == DT_F32 ? 4 : 2)) return DT_ERR_MISALIGNED;
+  hipStream_t s = dt::as_hip(stream);
+  if (scale_layout == DT_SCALE_BLOCKED) {
+    const int64_t SR = axis == 1 ? rows : cols, SC = (axis == 1 ? cols : rows) / 32;
+    if (SR % 128 != 0 || SC % 4 != 0) {  // zero the padding the cast itself never writes
+      const int64_t n = dt_blocked_scale_bytes(SR, SC);
+      dt::fill_bytes_kernel<<<(unsigned)std::min<int64_t>(dt::ceil_div(n, 256), 4096), 256, 0, s>>>(scale, n, 0);
+      if (int st = dt::launch_status()) return st;
+    }
+  }
+  MxArgs a{x, rows, cols, axis, transpose, static_cast<uint8_t*>(data), scale, s};
+  switch (in_dtype) {
+    case DT_F32: return launch_mx_in<DT_F32>(a, out_dtype, scale_layout);
+    case DT_BF16: return launch_mx_in<DT_BF16>(a, out_dtype, scale_layout);
+    default: return launch_mx_in<DT_F16>(a, out_dtype, scale_layout);
+  }
+}
+
+extern "C" int dt_to_blocked(const uint8_t* scale, int64_t R, int64_t C, uint8_t* out, dt_stream_t stream) {
+  if (R < 0 || C < 0) return DT_ERR_INVALID_SHAPE;
+  if (R == 0 || C == 0) return DT_OK;
+  if (!scale || !out) return DT_ERR_NULL_POINTER;
+  hipStream_t s = dt::as_hip(stream);
+  if (R % 128 != 0 || C % 4 != 0) {
+    const int64_t n = dt_blocked_scale_bytes(R, C);
+    dt::fill_bytes_kernel<<<(unsigned)std::min<int64_t>(dt::ceil_div(n, 256), 4096), 256, 0, s>>>(out, n, 0);
+    if (int st = dt::launch_status()) return st;
+  }
+  if (dt::ceil_div(R * C, 256) > 0x7FFFFFFFll) return DT_ERR_INVALID_SHAPE;
+  dt::to_blocked_kernel<<<(unsigned)dt::ceil_div(R * C, 256), 256, 0, s>>>(scale, R, C, out);
+  return dt::launch_status();
+}

@@ -1,0 +1,333 @@
+// MXFP8 cast kernels: one E8M0 scale byte per 32 elements plus the fp8 payload.
+//
+//  mx_row_kernel   blocks along rows.  A 32-element block is spread over 4 lanes (16-bit
+//                  input, 8 elements per 16-byte load) or 8 lanes (fp32 input); the block
+//                  maximum is an integer max over DPP quad/row permutes -- no LDS.
+//  mx_col_kernel   blocks down columns.  A lane owns 8 (fp32: 4) adjacent columns of a
+//                  32-row tile, so the block maximum needs no cross-lane traffic at all;
+//                  the payload is written in the input orientation or transposed.
+//  mx_any_kernel   one thread per block, arbitrary strides: covers every (axis, transpose)
+//                  pair and shapes the fast kernels do not take.
+#pragma once
+
+#include "dt_device.hpp"
+#include "dt_host.hpp"
+#include "quant_kernels.hpp"
+
+namespace dt {
+
+// position of scale (r, c) of an [R, C] scale matrix in the 128x4 blocked layout
+__host__ __device__ __forceinline__ int64_t blocked_offset(int64_t r, int64_t c, int64_t col_tiles /* ceil(C/4) */) {
+  return ((r >> 7) * col_tiles + (c >> 2)) * 512 + (r & 31) * 16 + ((r & 127) >> 5) * 4 + (c & 3);
+}
+
+template <int LAYOUT>
+__device__ __forceinline__ int64_t scale_offset(int64_t r, int64_t c, int64_t C) {
+  if constexpr (LAYOUT == DT_SCALE_BLOCKED)
+    return blocked_offset(r, c, (C + 3) >> 2);
+  else
+    return r * C + c;
+}
+
+// Block magnitude (fp32 bit pattern of max|x|, NaN patterns sort highest) -> E8M0 byte and
+// the fp32 multiplier 2^(127-byte) that scales the block into the fp8 range.
+template <int OUT>
+struct MxScale {
+  uint32_t byte;  // 0..254, or 255 for a block that holds a NaN
+  float mult;
+  bool nan;
+};
+template <int OUT>
+__device__ __forceinline__ MxScale<OUT> mx_scale_from_absbits(uint32_t absbits) {
+  constexpr int kTargetPow2 = OUT == DT_E5M2 ? 15 : 8;
+  const int be = (int)(absbits >> 23);
+  const int mant_nz = (absbits & 0x7FFFFFu) ? 1 : 0;
+  int e = be - 127 + mant_nz;                       // ceil(log2) from the exponent field
+  if (be == 0) e = absbits == 0 ? -128 : -126;      // zero / subnormal maxima
+  int b = e - kTargetPow2 + 127;
+  b = b < 0 ? 0 : (b > 254 ? 254 : b);
+  MxScale<OUT> r;
+  r.nan = absbits > 0x7F800000u;
+  r.byte = r.nan ? 255u : (uint32_t)b;
+  r.mult = as_f32((uint32_t)(254 - b) << 23);       // b <= 248 for any input, so never 2^-127
+  return r;
+}
+
+// saturating convert without the NaN patch (NaN blocks are overwritten wholesale)
+template <int OUT>
+__device__ __forceinline__ uint32_t pack4_finite(float p0, float p1, float p2, float p3) {
+  uint32_t w = cvt_pk<OUT, false>(clamp_fp8<OUT>(p0), clamp_fp8<OUT>(p1), 0u);
+  return cvt_pk<OUT, true>(clamp_fp8<OUT>(p2), clamp_fp8<OUT>(p3), w);
+}
+
+template <int IN>
+__device__ __forceinline__ float load_elem(const void* x, int64_t i) {
+  if constexpr (IN == DT_F32) return static_cast<const float*>(x)[i];
+  else if constexpr (IN == DT_BF16) return as_f32((uint32_t)static_cast<const uint16_t*>(x)[i] << 16);
+  else return (float)static_cast<const _Float16*>(x)[i];
+}
+
+// 8 consecutive 16-bit elements (one 16-byte vector) as floats
+template <int IN>
+__device__ __forceinline__ void unpack8(u32x4 w, float (&f)[8]) {
+  if constexpr (IN == DT_BF16) {
+    f[0] = bf16_lo(w.x); f[1] = bf16_hi(w.x); f[2] = bf16_lo(w.y); f[3] = bf16_hi(w.y);
+    f[4] = bf16_lo(w.z); f[5] = bf16_hi(w.z); f[6] = bf16_lo(w.w); f[7] = bf16_hi(w.w);
+  } else {
+    f[0] = f16_lo(w.x); f[1] = f16_hi(w.x); f[2] = f16_lo(w.y); f[3] = f16_hi(w.y);
+    f[4] = f16_lo(w.z); f[5] = f16_hi(w.z); f[6] = f16_lo(w.w); f[7] = f16_hi(w.w);
+  }
+}
+
+// fp32 bit pattern of the largest magnitude in one 16-byte vector
+template <int IN>
+__device__ __forceinline__ uint32_t vec_absmax_bits(u32x4 w) {
+  if constexpr (IN == DT_F32) {
+    return umax(umax(absbits_f32(w.x), absbits_f32(w.y)), umax(absbits_f32(w.z), absbits_f32(w.w)));
+  } else if constexpr (IN == DT_BF16) {
+    uint32_t p = pk_absmax16(pk_absmax16(pk_absmax16(pk_absmax16(0u, w.x), w.y), w.z), w.w);
+    return umax(p & 0xFFFFu, p >> 16) << 16;
+  } else {
+    float f[8];
+    unpack8<IN>(w, f);
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) m = umax(m, absbits_f32(as_u32(f[i])));
+    return m;
+  }
+}
+
+// ------------------------------------------------------------------ blocks along rows
+// The matrix is a flat run of 32-element blocks.  One wave pass ("super-chunk") covers 64
+// blocks as LPB chunks of 64 vectors; lane l ends up holding the scale byte of chunk
+// l % LPB, block l / LPB, so the 64 scale bytes leave in a single store instruction.
+template <int IN, int OUT, int LAYOUT>
+__global__ __launch_bounds__(kBlock) void mx_row_kernel(const void* __restrict__ x, uint32_t nblocks,
+                                                        uint32_t kblocks, uint8_t* __restrict__ data,
+                                                        uint8_t* __restrict__ scale) {
+  constexpr int kV = InTraits<IN>::kVec;      // elements per vector
+  constexpr int LPB = 32 / kV;                // lanes per block: 4 or 8
+  constexpr int BPC = kWave / LPB;            // blocks per chunk: 16 or 8
+  const int lane = threadIdx.x % kWave;
+  const uint32_t nvec = nblocks * LPB;
+  const u32x4* v = static_cast<const u32x4*>(x);
+  const uint32_t nsuper = (nblocks + 63u) / 64u;
+  const uint32_t wave_id = (blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const uint32_t nwaves = gridDim.x * (kBlock / kWave);
+
+  for (uint32_t sc = wave_id; sc < nsuper; sc += nwaves) {
+    const uint32_t vbase = sc * 64u * LPB + lane;
+    u32x4 w[LPB];
+#pragma unroll
+    for (int c = 0; c < LPB; ++c) {
+      const uint32_t vi = vbase + c * kWave;
+      w[c] = vi < nvec ? v[vi] : u32x4{0u, 0u, 0u, 0u};
+    }
+    uint32_t mybyte = 0;
+#pragma unroll
+    for (int c = 0; c < LPB; ++c) {
+      const uint32_t vi = vbase + c * kWave;
+      uint32_t m = quad_umax(vec_absmax_bits<IN>(w[c]));
+      if constexpr (LPB == 8) m = umax(m, dpp<kDppRowHalfMirror>(m));
+      const MxScale<OUT> s = mx_scale_from_absbits<OUT>(m);
+      if ((lane % LPB) == c) mybyte = s.byte;
+      if (vi < nvec) {
+        if constexpr (IN == DT_F32) {
+          uint32_t r = pack4_finite<OUT>(as_f32(w[c].x) * s.mult, as_f32(w[c].y) * s.mult, as_f32(w[c].z) * s.mult,
+                                         as_f32(w[c].w) * s.mult);
+          reinterpret_cast<uint32_t*>(data)[vi] = s.nan ? 0x7F7F7F7Fu : r;
+        } else {
+          float f[8];
+          unpack8<IN>(w[c], f);
+          u32x2 r;
+          r.x = pack4_finite<OUT>(f[0] * s.mult, f[1] * s.mult, f[2] * s.mult, f[3] * s.mult);
+          r.y = pack4_finite<OUT>(f[4] * s.mult, f[5] * s.mult, f[6] * s.mult, f[7] * s.mult);
+          if (s.nan) r = u32x2{0x7F7F7F7Fu, 0x7F7F7F7Fu};
+          reinterpret_cast<u32x2*>(data)[vi] = r;
+        }
+      }
+    }
+    const uint32_t g = sc * 64u + (lane % LPB) * BPC + lane / LPB;  // block index of mybyte
+    if (g < nblocks) {
+      if constexpr (LAYOUT == DT_SCALE_BLOCKED) {
+        const uint32_t r = g / kblocks, c = g - r * kblocks;
+        scale[blocked_offset(r, c, (kblocks + 3) >> 2)] = (uint8_t)mybyte;
+      } else {
+        scale[g] = (uint8_t)mybyte;
+      }
+    }
+  }
+}
+
+// --------------------------------------------------------------- blocks down columns
+// One wave owns RBW consecutive 32-row tiles of 64*kV columns.  TRANSPOSE writes the payload
+// as [cols, rows] (32 contiguous bytes per column and tile) and the scales as
+// [cols, rows/32]; otherwise payload [rows, cols] and scales [rows/32, cols].
+template <int IN, int OUT, bool TRANSPOSE, int LAYOUT, int RBW>
+__global__ __launch_bounds__(kBlock) void mx_col_kernel(const void* __restrict__ x, uint32_t rows, uint32_t cols,
+                                                        uint8_t* __restrict__ data, uint8_t* __restrict__ scale) {
+  constexpr int kV = InTraits<IN>::kVec;   // columns per lane
+  constexpr int kW = kV / 4;               // fp8 words per lane and row: 2 or 1
+  const int lane = threadIdx.x % kWave;
+  const uint32_t row_tiles = rows / 32u, rb_groups = (row_tiles + RBW - 1) / RBW;
+  const uint32_t col_tiles = (cols + kWave * kV - 1) / (kWave * kV);
+  const uint32_t wave_id = (blockIdx.x * kBlock + threadIdx.x) / kWave;
+  if (wave_id >= rb_groups * col_tiles) return;  // whole wave leaves; no barrier in this kernel
+  // consecutive waves walk down the rows first so a workgroup covers adjacent row tiles
+  const uint32_t ct = wave_id / rb_groups, rg = wave_id - ct * rb_groups;
+  const uint32_t col0 = ct * (kWave * kV) + lane * kV;
+  if (col0 >= cols) return;  // cols % kV == 0, so a lane is either fully inside or outside
+  const uint32_t row_vecs = cols / kV;
+  const u32x4* v = static_cast<const u32x4*>(x);
+  uint32_t sbytes[kV];  // per column: RBW scale bytes packed (TRANSPOSE only)
+#pragma unroll
+  for (int c = 0; c < kV; ++c) sbytes[c] = 0;
+
+#pragma unroll
+  for (int t = 0; t < RBW; ++t) {
+    const uint32_t rb = rg * RBW + t;
+    if (rb >= row_tiles) break;
+    const uint64_t vfirst = (uint64_t)rb * 32u * row_vecs + col0 / kV;
+    u32x4 w[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) w[i] = v[vfirst + (uint64_t)i * row_vecs];
+
+    // per-column magnitude maxima
+    uint32_t cm[kV];
+    if constexpr (IN == DT_BF16) {
+      uint32_t p0 = 0, p1 = 0, p2 = 0, p3 = 0;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) {
+        p0 = pk_absmax16(p0, w[i].x); p1 = pk_absmax16(p1, w[i].y);
+        p2 = pk_absmax16(p2, w[i].z); p3 = pk_absmax16(p3, w[i].w);
+      }
+      cm[0] = p0 << 16; cm[1] = p0 & 0xFFFF0000u; cm[2] = p1 << 16; cm[3] = p1 & 0xFFFF0000u;
+      cm[4] = p2 << 16; cm[5] = p2 & 0xFFFF0000u; cm[6] = p3 << 16; cm[7] = p3 & 0xFFFF0000u;
+    } else if constexpr (IN == DT_F16) {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) cm[c] = 0;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) {
+        float f[8];
+        unpack8<IN>(w[i], f);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) cm[c] = umax(cm[c], absbits_f32(as_u32(f[c])));
+      }
+    } else {
+      cm[0] = cm[1] = cm[2] = cm[3] = 0;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) {
+        cm[0] = umax(cm[0], absbits_f32(w[i].x)); cm[1] = umax(cm[1], absbits_f32(w[i].y));
+        cm[2] = umax(cm[2], absbits_f32(w[i].z)); cm[3] = umax(cm[3], absbits_f32(w[i].w));
+      }
+    }
+    float mult[kV];
+    bool nanc[kV];
+    uint32_t byte_lo = 0, byte_hi = 0;  // the kV scale bytes packed in column order
+#pragma unroll
+    for (int c = 0; c < kV; ++c) {
+      const MxScale<OUT> s = mx_scale_from_absbits<OUT>(cm[c]);
+      mult[c] = s.mult;
+      nanc[c] = s.nan;
+      if (c < 4) byte_lo |= s.byte << (8 * c); else byte_hi |= s.byte << (8 * (c - 4));
+      sbytes[c] |= s.byte << (8 * t);
+    }
+    auto elem = [&](int i, int c) -> float {
+      if constexpr (IN == DT_F32) {
+        return as_f32(c == 0 ? w[i].x : c == 1 ? w[i].y : c == 2 ? w[i].z : w[i].w);
+      } else {
+        const uint32_t d = (c >> 1) == 0 ? w[i].x : (c >> 1) == 1 ? w[i].y : (c >> 1) == 2 ? w[i].z : w[i].w;
+        if constexpr (IN == DT_BF16) return (c & 1) ? bf16_hi(d) : bf16_lo(d);
+        else return (c & 1) ? f16_hi(d) : f16_lo(d);
+      }
+    };
+    if constexpr (!TRANSPOSE) {
+      uint8_t* drow = data + (uint64_t)rb * 32u * cols + col0;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) {
+        uint32_t r[kW];
+#pragma unroll
+        for (int q = 0; q < kW; ++q) {
+          r[q] = pack4_finite<OUT>(elem(i, 4 * q) * mult[4 * q], elem(i, 4 * q + 1) * mult[4 * q + 1],
+                                   elem(i, 4 * q + 2) * mult[4 * q + 2], elem(i, 4 * q + 3) * mult[4 * q + 3]);
+          uint32_t nanmask = (nanc[4 * q] ? 0xFFu : 0u) | (nanc[4 * q + 1] ? 0xFF00u : 0u) |
+                             (nanc[4 * q + 2] ? 0xFF0000u : 0u) | (nanc[4 * q + 3] ? 0xFF000000u : 0u);
+          r[q] = (r[q] & ~nanmask) | (0x7F7F7F7Fu & nanmask);
+        }
+        if constexpr (kW == 2) *reinterpret_cast<u32x2*>(drow + (uint64_t)i * cols) = u32x2{r[0], r[1]};
+        else *reinterpret_cast<uint32_t*>(drow + (uint64_t)i * cols) = r[0];
+      }
+      // scales [rows/32, cols]: kV adjacent bytes
+      uint8_t* srow = scale + (uint64_t)rb * cols + col0;
+      if constexpr (kW == 2) *reinterpret_cast<u32x2*>(srow) = u32x2{byte_lo, byte_hi};
+      else *reinterpret_cast<uint32_t*>(srow) = byte_lo;
+    } else {
+#pragma unroll
+      for (int c = 0; c < kV; ++c) {
+        uint32_t r[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          r[q] = pack4_finite<OUT>(elem(4 * q, c) * mult[c], elem(4 * q + 1, c) * mult[c],
+                                   elem(4 * q + 2, c) * mult[c], elem(4 * q + 3, c) * mult[c]);
+          if (nanc[c]) r[q] = 0x7F7F7F7Fu;
+        }
+        u32x4* dcol = reinterpret_cast<u32x4*>(data + (uint64_t)(col0 + c) * rows + (uint64_t)rb * 32u);
+        dcol[0] = u32x4{r[0], r[1], r[2], r[3]};
+        dcol[1] = u32x4{r[4], r[5], r[6], r[7]};
+      }
+    }
+  }
+  if constexpr (TRANSPOSE) {
+    // scales [cols, rows/32]: this wave's RBW bytes per column are adjacent
+    const uint32_t rb0 = rg * RBW;
+#pragma unroll
+    for (int c = 0; c < kV; ++c) {
+#pragma unroll
+      for (int t = 0; t < RBW; ++t) {
+        if (rb0 + t < row_tiles)
+          scale[scale_offset<LAYOUT>(col0 + c, rb0 + t, row_tiles)] = (uint8_t)(sbytes[c] >> (8 * t));
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------------- any orientation ---
+// One thread per 32-element block with explicit strides (in elements / bytes).
+template <int IN, int OUT, int LAYOUT>
+__global__ __launch_bounds__(kBlock) void mx_any_kernel(const void* __restrict__ x, int64_t outer, int64_t inner_blocks,
+                                                        int64_t x_outer_stride, int64_t x_elem_stride,
+                                                        int64_t d_outer_stride, int64_t d_elem_stride,
+                                                        int64_t s_rows, int64_t s_cols, int s_transposed,
+                                                        uint8_t* __restrict__ data, uint8_t* __restrict__ scale) {
+  const int64_t g = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (g >= outer * inner_blocks) return;
+  const int64_t o = g / inner_blocks, b = g - o * inner_blocks;
+  const int64_t xfirst = o * x_outer_stride + b * 32 * x_elem_stride;
+  uint32_t m = 0;
+  for (int i = 0; i < 32; ++i) m = umax(m, absbits_f32(as_u32(load_elem<IN>(x, xfirst + i * x_elem_stride))));
+  const MxScale<OUT> s = mx_scale_from_absbits<OUT>(m);
+  const int64_t dfirst = o * d_outer_stride + b * 32 * d_elem_stride;
+  for (int i = 0; i < 32; ++i) {
+    const float p = load_elem<IN>(x, xfirst + i * x_elem_stride) * s.mult;
+    const uint32_t code = pack4_finite<OUT>(p, 0.f, 0.f, 0.f) & 0xFFu;
+    data[dfirst + i * d_elem_stride] = s.nan ? (uint8_t)0x7F : (uint8_t)code;
+  }
+  // the scale matrix is [outer, inner_blocks], stored transposed when s_transposed
+  const int64_t sr = s_transposed ? b : o, scol = s_transposed ? o : b;
+  scale[scale_offset<LAYOUT>(sr, scol, s_cols)] = (uint8_t)s.byte;
+  (void)s_rows;
+}
+
+__global__ void fill_bytes_kernel(uint8_t* p, int64_t n, uint8_t value) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = value;
+}
+
+// plain [R, C] scale matrix -> blocked layout (padding already zeroed by the caller)
+__global__ void to_blocked_kernel(const uint8_t* __restrict__ in, int64_t R, int64_t C, uint8_t* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= R * C) return;
+  const int64_t r = i / C, c = i - r * C;
+  out[blocked_offset(r, c, (C + 3) >> 2)] = in[i];
+}
+
+}  // namespace dt

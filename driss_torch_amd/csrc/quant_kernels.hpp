@@ -1,0 +1,299 @@
+// Kernel templates of the per-tensor path: the amax reduction and the saturating fp8 cast.
+// Both stream the tensor with 16-byte loads from a persistent grid; they are shared by
+// amax.hip, saturated_cast.hip and dynamic_scaled_quant.hip.
+#pragma once
+
+#include "dt_device.hpp"
+#include "dt_host.hpp"
+
+namespace dt {
+
+constexpr int kBlock = 256;  // 4 waves
+
+template <int IN>
+struct InTraits;
+template <>
+struct InTraits<DT_F32> {
+  static constexpr int kBytes = 4, kVec = 4;  // elements per 16-byte vector
+};
+template <>
+struct InTraits<DT_BF16> {
+  static constexpr int kBytes = 2, kVec = 8;
+};
+template <>
+struct InTraits<DT_F16> {
+  static constexpr int kBytes = 2, kVec = 8;
+};
+
+// How a flat tensor is cut for 16-byte access: `head` leading elements up to the first
+// aligned address, `nvec` whole vectors, `tail` trailing elements.
+struct Split {
+  int64_t head, nvec, tail;
+};
+template <int IN>
+inline Split split_for_vectors(const void* x, int64_t numel) {
+  constexpr int kB = InTraits<IN>::kBytes, kV = InTraits<IN>::kVec;
+  uintptr_t mis = reinterpret_cast<uintptr_t>(x) % 16;
+  int64_t head = mis ? (int64_t)((16 - mis) / kB) : 0;
+  if (head > numel) head = numel;
+  int64_t nvec = (numel - head) / kV;
+  return {head, nvec, numel - head - nvec * kV};
+}
+
+template <int IN>
+__device__ __forceinline__ uint32_t absbits_of(const void* x, int64_t i) {
+  if constexpr (IN == DT_F32)
+    return static_cast<const uint32_t*>(x)[i] & 0x7FFFFFFFu;
+  else
+    return ((uint32_t)static_cast<const uint16_t*>(x)[i] & 0x7FFFu) << 16;  // bf16 -> f32 bits
+}
+
+// --------------------------------------------------------------------------- amax ----
+// Every workgroup reduces a grid-strided share of the vectors to one unsigned magnitude,
+// publishes it in the workspace and takes a ticket; the workgroup that draws the last
+// ticket reduces the partials, writes amax (and, when NSCALES > 0, the fp8 scales derived
+// from it) and re-arms the ticket for the next launch.
+template <int IN, int UNROLL, int NSCALES>
+__global__ __launch_bounds__(kBlock) void amax_kernel(const void* __restrict__ x, Split sp,
+                                                      uint8_t* __restrict__ ws, float* __restrict__ amax_out,
+                                                      float* __restrict__ scale_out, float fmax0, float fmax1) {
+  constexpr int kB = InTraits<IN>::kBytes, kV = InTraits<IN>::kVec;
+  __shared__ uint32_t lds[kBlock / kWave];
+  __shared__ uint32_t is_last;
+  const int tid = threadIdx.x;
+  const u32x4* v = reinterpret_cast<const u32x4*>(static_cast<const uint8_t*>(x) + sp.head * kB);
+
+  uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+  auto absorb = [&](u32x4 w) {
+    if constexpr (IN == DT_F32) {
+      a0 = umax(a0, absbits_f32(w.x)); a1 = umax(a1, absbits_f32(w.y));
+      a2 = umax(a2, absbits_f32(w.z)); a3 = umax(a3, absbits_f32(w.w));
+    } else {
+      a0 = pk_absmax16(a0, w.x); a1 = pk_absmax16(a1, w.y);
+      a2 = pk_absmax16(a2, w.z); a3 = pk_absmax16(a3, w.w);
+    }
+  };
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  int64_t i = (int64_t)blockIdx.x * kBlock + tid;
+  for (; i + (UNROLL - 1) * stride < sp.nvec; i += UNROLL * stride) {
+    u32x4 w[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) w[u] = v[i + u * stride];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) absorb(w[u]);
+  }
+  for (; i < sp.nvec; i += stride) absorb(v[i]);
+
+  uint32_t m;
+  if constexpr (IN == DT_F32) {
+    m = umax(umax(a0, a1), umax(a2, a3));
+  } else {
+    uint32_t p = pk_absmax16(pk_absmax16(a0, a1), pk_absmax16(a2, a3));
+    m = umax(p & 0xFFFFu, p >> 16) << 16;
+  }
+  if (blockIdx.x == 0) {  // the few elements outside the aligned body
+    if (tid < sp.head) m = umax(m, absbits_of<IN>(x, tid));
+    if (tid < sp.tail) m = umax(m, absbits_of<IN>(x, sp.head + sp.nvec * kV + tid));
+  }
+  m = block_umax<kBlock / kWave>(m, lds);
+
+  uint32_t* ticket = reinterpret_cast<uint32_t*>(ws + kWsTicket);
+  uint32_t* partials = reinterpret_cast<uint32_t*>(ws + kWsPartials);
+  if (tid == 0) {
+    __hip_atomic_store(&partials[blockIdx.x], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __threadfence();  // publish the partial before the ticket
+    uint32_t t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    is_last = (t == gridDim.x - 1) ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!is_last) return;
+
+  __threadfence();
+  uint32_t r = 0;
+  for (int j = tid; j < (int)gridDim.x; j += kBlock)
+    r = umax(r, __hip_atomic_load(&partials[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  r = block_umax<kBlock / kWave>(r, lds);
+  if (tid == 0) {
+    const float amax = as_f32(r);
+    *reinterpret_cast<float*>(ws + kWsAmax) = amax;
+    if (amax_out) *amax_out = amax;
+    if constexpr (NSCALES > 0) {
+      float* wscale = reinterpret_cast<float*>(ws + kWsScale);
+      const float s0 = amax_to_scale(amax, fmax0);
+      wscale[0] = s0;
+      if (scale_out) scale_out[0] = s0;
+      if constexpr (NSCALES > 1) {
+        const float s1 = amax_to_scale(amax, fmax1);
+        wscale[1] = s1;
+        if (scale_out) scale_out[1] = s1;
+      }
+    }
+    __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // re-arm
+  }
+}
+
+inline int reduction_grid(int64_t nvec, int unroll, const char* knob) {
+  int64_t want = ceil_div(nvec, (int64_t)kBlock * unroll);
+  int64_t cap = (int64_t)device_facts().cu_count * tuning(knob);
+  if (cap > kMaxPartials) cap = kMaxPartials;
+  if (want > cap) want = cap;
+  return want < 1 ? 1 : (int)want;
+}
+
+// Enqueue the amax reduction.  nscales: 0 = amax only, 1 = scale for fmax0, 2 = both.
+template <int IN>
+inline int launch_amax(const void* x, int64_t numel, void* ws, float* amax_out, float* scale_out, int nscales,
+                       float fmax0, float fmax1, hipStream_t stream) {
+  constexpr int kUnroll = 8;
+  Split sp = split_for_vectors<IN>(x, numel);
+  int grid = reduction_grid(sp.nvec, kUnroll, "amax.blocks_per_cu");
+  uint8_t* w = static_cast<uint8_t*>(ws);
+  if (nscales == 0)
+    amax_kernel<IN, kUnroll, 0><<<grid, kBlock, 0, stream>>>(x, sp, w, amax_out, scale_out, fmax0, fmax1);
+  else if (nscales == 1)
+    amax_kernel<IN, kUnroll, 1><<<grid, kBlock, 0, stream>>>(x, sp, w, amax_out, scale_out, fmax0, fmax1);
+  else
+    amax_kernel<IN, kUnroll, 2><<<grid, kBlock, 0, stream>>>(x, sp, w, amax_out, scale_out, fmax0, fmax1);
+  return launch_status();
+}
+
+// --------------------------------------------------------------------------- cast ----
+// ROUND_BF16: round the product to bf16 before the convert (modes 1 and 2 of
+// dt_round_mode, bf16 input only); ROUND_SCALE: also round the scale itself (mode 2).
+template <int IN, int OUT, bool ROUND_BF16>
+__device__ __forceinline__ void cast_vec(u32x4 w, float s, uint8_t* __restrict__ out, int64_t vec_index) {
+  if constexpr (IN == DT_F32) {
+    uint32_t r = pack4<OUT>(scaled<false>(as_f32(w.x), s), scaled<false>(as_f32(w.y), s),
+                            scaled<false>(as_f32(w.z), s), scaled<false>(as_f32(w.w), s));
+    reinterpret_cast<uint32_t*>(out)[vec_index] = r;
+  } else {
+    u32x2 r;
+    r.x = pack4<OUT>(scaled<ROUND_BF16>(bf16_lo(w.x), s), scaled<ROUND_BF16>(bf16_hi(w.x), s),
+                     scaled<ROUND_BF16>(bf16_lo(w.y), s), scaled<ROUND_BF16>(bf16_hi(w.y), s));
+    r.y = pack4<OUT>(scaled<ROUND_BF16>(bf16_lo(w.z), s), scaled<ROUND_BF16>(bf16_hi(w.z), s),
+                     scaled<ROUND_BF16>(bf16_lo(w.w), s), scaled<ROUND_BF16>(bf16_hi(w.w), s));
+    reinterpret_cast<u32x2*>(out)[vec_index] = r;
+  }
+}
+
+template <int IN, int OUT, bool ROUND_BF16>
+__device__ __forceinline__ uint8_t cast_one(const void* x, int64_t i, float s) {
+  float xv;
+  if constexpr (IN == DT_F32)
+    xv = static_cast<const float*>(x)[i];
+  else
+    xv = as_f32((uint32_t)static_cast<const uint16_t*>(x)[i] << 16);
+  return (uint8_t)(pack4<OUT>(scaled<ROUND_BF16>(xv, s), 0.f, 0.f, 0.f) & 0xFFu);
+}
+
+// Aligned streaming cast: x 16-byte aligned, out aligned to its packed store.  The tail
+// (< one vector) is done by the first workgroup.  With PAIR the same read also feeds a
+// second output of the other fp8 type with its own scale (scale[1], out2).
+template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR, int UNROLL>
+__global__ __launch_bounds__(kBlock) void cast_kernel(const void* __restrict__ x, int64_t nvec, int64_t tail,
+                                                      const float* __restrict__ scale, uint8_t* __restrict__ out,
+                                                      uint8_t* __restrict__ out2) {
+  constexpr int kV = InTraits<IN>::kVec;
+  constexpr int OUT2 = OUT == DT_E4M3FN ? DT_E5M2 : DT_E4M3FN;
+  float s = scale[0], s2 = PAIR ? scale[1] : 0.f;
+  if constexpr (ROUND_SCALE) { s = round_to_bf16(s); s2 = round_to_bf16(s2); }
+  const u32x4* v = static_cast<const u32x4*>(x);
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  for (; i + (UNROLL - 1) * stride < nvec; i += UNROLL * stride) {
+    u32x4 w[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) w[u] = v[i + u * stride];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      cast_vec<IN, OUT, ROUND_BF16>(w[u], s, out, i + u * stride);
+      if constexpr (PAIR) cast_vec<IN, OUT2, ROUND_BF16>(w[u], s2, out2, i + u * stride);
+    }
+  }
+  for (; i < nvec; i += stride) {
+    u32x4 w = v[i];
+    cast_vec<IN, OUT, ROUND_BF16>(w, s, out, i);
+    if constexpr (PAIR) cast_vec<IN, OUT2, ROUND_BF16>(w, s2, out2, i);
+  }
+  if (blockIdx.x == 0 && threadIdx.x < tail) {
+    const int64_t e = nvec * kV + threadIdx.x;
+    out[e] = cast_one<IN, OUT, ROUND_BF16>(x, e, s);
+    if constexpr (PAIR) out2[e] = cast_one<IN, OUT2, ROUND_BF16>(x, e, s2);
+  }
+}
+
+// Any alignment: one element per thread per step.
+template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR>
+__global__ __launch_bounds__(kBlock) void cast_kernel_unaligned(const void* __restrict__ x, int64_t numel,
+                                                                const float* __restrict__ scale,
+                                                                uint8_t* __restrict__ out, uint8_t* __restrict__ out2) {
+  constexpr int OUT2 = OUT == DT_E4M3FN ? DT_E5M2 : DT_E4M3FN;
+  float s = scale[0], s2 = PAIR ? scale[1] : 0.f;
+  if constexpr (ROUND_SCALE) { s = round_to_bf16(s); s2 = round_to_bf16(s2); }
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < numel; i += stride) {
+    out[i] = cast_one<IN, OUT, ROUND_BF16>(x, i, s);
+    if constexpr (PAIR) out2[i] = cast_one<IN, OUT2, ROUND_BF16>(x, i, s2);
+  }
+}
+
+template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR>
+inline int launch_cast_impl(const void* x, int64_t numel, const float* scale, void* out, void* out2,
+                            hipStream_t stream) {
+  constexpr int kUnroll = 4;
+  constexpr size_t kStoreAlign = IN == DT_F32 ? 4 : 8;
+  uint8_t* o = static_cast<uint8_t*>(out);
+  uint8_t* o2 = static_cast<uint8_t*>(out2);
+  const bool fast = aligned(x, 16) && aligned(out, kStoreAlign) && (!PAIR || aligned(out2, kStoreAlign));
+  if (fast) {
+    const int64_t nvec = numel / InTraits<IN>::kVec, tail = numel % InTraits<IN>::kVec;
+    int grid = reduction_grid(nvec, kUnroll, "cast.blocks_per_cu");
+    cast_kernel<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR, kUnroll><<<grid, kBlock, 0, stream>>>(x, nvec, tail, scale, o, o2);
+  } else {
+    int grid = reduction_grid(numel, 1, "cast.blocks_per_cu");
+    cast_kernel_unaligned<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR><<<grid, kBlock, 0, stream>>>(x, numel, scale, o, o2);
+  }
+  return launch_status();
+}
+
+// Runtime (in_dtype, out_dtype, round_mode) -> template instance.  `pair` adds out2 of the
+// other fp8 type with scale[1].
+template <bool PAIR>
+inline int launch_cast(const void* x, int in_dtype, int64_t numel, const float* scale, int out_dtype,
+                       int round_mode, void* out, void* out2, hipStream_t stream) {
+#define DT_CAST(IN, OUT, RB, RS) return launch_cast_impl<IN, OUT, RB, RS, PAIR>(x, numel, scale, out, out2, stream)
+  if (in_dtype == DT_F32) {
+    if (out_dtype == DT_E4M3FN) DT_CAST(DT_F32, DT_E4M3FN, false, false);
+    DT_CAST(DT_F32, DT_E5M2, false, false);
+  }
+  if (round_mode == DT_ROUND_F32) {
+    if (out_dtype == DT_E4M3FN) DT_CAST(DT_BF16, DT_E4M3FN, false, false);
+    DT_CAST(DT_BF16, DT_E5M2, false, false);
+  }
+  if (round_mode == DT_ROUND_BF16_PRODUCT) {
+    if (out_dtype == DT_E4M3FN) DT_CAST(DT_BF16, DT_E4M3FN, true, false);
+    DT_CAST(DT_BF16, DT_E5M2, true, false);
+  }
+  if (out_dtype == DT_E4M3FN) DT_CAST(DT_BF16, DT_E4M3FN, true, true);
+  DT_CAST(DT_BF16, DT_E5M2, true, true);
+#undef DT_CAST
+}
+
+inline int check_cast_args(const void* x, int in_dtype, int64_t numel, int out_dtype, int round_mode, const void* out) {
+  if (in_dtype != DT_F32 && in_dtype != DT_BF16) return DT_ERR_INVALID_DTYPE;
+  if (out_dtype != DT_E4M3FN && out_dtype != DT_E5M2) return DT_ERR_INVALID_DTYPE;
+  if (round_mode < DT_ROUND_BF16_PRODUCT || round_mode > DT_ROUND_F32) return DT_ERR_INVALID_MODE;
+  if (numel < 0) return DT_ERR_INVALID_SHAPE;
+  if (numel > 0 && (!x || !out)) return DT_ERR_NULL_POINTER;
+  if (!aligned(x, in_dtype == DT_F32 ? 4 : 2)) return DT_ERR_MISALIGNED;
+  return DT_OK;
+}
+
+inline int check_workspace(const void* ws, size_t bytes) {
+  if (!ws) return DT_ERR_WORKSPACE;
+  if (bytes < kWsBytes) return DT_ERR_WORKSPACE;
+  if (!aligned(ws, 256)) return DT_ERR_MISALIGNED;
+  return DT_OK;
+}
+
+}  // namespace dt

@@ -1,0 +1,179 @@
+/*
+ * driss_torch_hip.h -- C ABI of the MI355X (gfx950) FP8 / MX quantization kernels.
+ *
+ * Plain pointers and sizes only: no torch types, no C++ types, no exceptions.  Every entry
+ * point validates its arguments on the host, enqueues its kernels on `stream` (NULL = the
+ * legacy default stream), never synchronises, never allocates, and returns a dt_status
+ * code.  All data pointers are device pointers on the current HIP device.
+ *
+ * Each declaration cites the reference (drisspg/driss_torch) interface it stands in for;
+ * paths are relative to the reference tree.  The torch-facing registration shim
+ * (driss_torch_amd/csrc/register_ops.cpp) keeps the TORCH_LIBRARY(DrissTorch) schemas of
+ * src/register_ops.cpp:13-43 and calls only these functions.
+ */
+#ifndef DRISS_TORCH_HIP_H
+#define DRISS_TORCH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DT_API __attribute__((visibility("default")))
+
+/* hipStream_t without pulling in the HIP headers */
+typedef struct ihipStream_t* dt_stream_t;
+
+enum dt_status {
+  DT_OK = 0,
+  DT_ERR_INVALID_DTYPE = 1,   /* in/out dtype code not supported by this entry point */
+  DT_ERR_INVALID_SHAPE = 2,   /* negative size, or a divisibility requirement not met */
+  DT_ERR_NULL_POINTER = 3,
+  DT_ERR_MISALIGNED = 4,      /* pointer alignment requirement not met */
+  DT_ERR_WORKSPACE = 5,       /* workspace missing or too small */
+  DT_ERR_INVALID_MODE = 6,    /* round_mode / axis / layout code out of range */
+  DT_ERR_LAUNCH = 7,          /* hipGetLastError() after the launch was not hipSuccess */
+  DT_ERR_EMPTY = 8            /* reduction over zero elements */
+};
+
+/* element types of the high-precision operand */
+enum dt_in_dtype { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2 };
+/* OCP FP8 output types */
+enum dt_out_dtype { DT_E4M3FN = 0, DT_E5M2 = 1 };
+
+/*
+ * How the product x*scale is rounded for a bf16 `x` before the fp8 convert (fp32 input:
+ * the three coincide).  These are the three answers eager PyTorch gives for
+ * test/test_sat_cast.py:7-24 depending on the scale tensor:
+ *   DT_ROUND_BF16_PRODUCT        bf16(f32(x) * s)              0-dim CPU scale
+ *   DT_ROUND_BF16_SCALE_PRODUCT  bf16(f32(x) * f32(bf16(s)))   0-dim device scale; what the
+ *                                                              reference kernel computes,
+ *                                                              src/saturated_cast.cu:66,81
+ *   DT_ROUND_F32                 f32(x) * s                    scale of rank >= 1
+ */
+enum dt_round_mode { DT_ROUND_BF16_PRODUCT = 1, DT_ROUND_BF16_SCALE_PRODUCT = 2, DT_ROUND_F32 = 3 };
+
+/* layout of the E8M0 scale bytes written by dt_mx_fp8_quantize */
+enum dt_scale_layout {
+  DT_SCALE_PLAIN = 0,   /* row-major [rows, blocks]: what src/mx_cast.cu:197-199,210-211 emits */
+  DT_SCALE_BLOCKED = 1  /* 128x4 interleaved tiles: what src/mx_fp8_bf16.cu:197-205 consumes */
+};
+
+DT_API const char* dt_status_string(int status);
+DT_API int dt_abi_version(void);
+
+/* ------------------------------------------------------------------ workspace --------
+ * dt_amax and dt_dynamic_scaled_quant combine per-workgroup partial maxima through a
+ * small device workspace (partials + an arrival counter).  The caller owns it: allocate
+ * dt_workspace_bytes() bytes (256-byte aligned), call dt_workspace_init once, then reuse
+ * it for any number of calls that are ordered on one stream.  Calls that may overlap on
+ * the device need separate workspaces.  (The reference allocates its scratch per call
+ * from the torch allocator: src/amax.cu:115, src/dynamic_scaled_quant.cu:172.)          */
+DT_API size_t dt_workspace_bytes(void);
+DT_API int dt_workspace_init(void* workspace, size_t workspace_bytes, dt_stream_t stream);
+
+/* ------------------------------------------------------------------ amax -------------
+ * out[0] = max_i |x_i| as fp32 (NaN if any x_i is NaN).  Replaces driss_torch::amax,
+ * src/amax.cu:106-119 (host) and :70-102 (kernel + launch).  x: DT_F32 or DT_BF16, any
+ * numel >= 1 (the reference needs an even numel, src/amax.cu:113), any alignment of the
+ * element type.                                                                          */
+DT_API int dt_amax(const void* x, int in_dtype, int64_t numel, float* out, void* workspace,
+                   size_t workspace_bytes, dt_stream_t stream);
+
+/* ------------------------------------------------------------ saturated_cast ---------
+ * out[i] = fp8_rne(clamp(x[i] * scale[0], -fmax, fmax)), NaN kept.  Replaces
+ * driss_torch::saturated_cast, src/saturated_cast.cu:227-252 (host), :168-224 (dispatch),
+ * :38-153 (kernels).  `scale` is one fp32 value in device memory.  The elements are taken
+ * in storage order, so a column-major input gives a column-major output exactly as
+ * src/saturated_cast.cu:243-249 does.  numel >= 0.                                       */
+DT_API int dt_saturated_cast(const void* x, int in_dtype, int64_t numel, const float* scale,
+                             int out_dtype, int round_mode, void* out, dt_stream_t stream);
+
+/* -------------------------------------------------------- dynamic_scaled_quant -------
+ * Per tensor: amax = max|x|, scale = f32(fmax / max(f64(amax), 1e-12)), out as
+ * dt_saturated_cast.  Replaces driss_torch::dynamic_scaled_quant,
+ * src/dynamic_scaled_quant.cu:157-176 (host), :119-153 (launch), :83-118 (kernel); the
+ * scale formula is the one its test checks, test/test_dynamic_quant.py:36 (the kernel's
+ * own `fmax / (amax + 1e-12)` at :111 differs in the last bits).  amax_out / scale_out may
+ * be NULL.  The reference runs fp32 input only (:130,135); bf16 is accepted here.        */
+DT_API int dt_dynamic_scaled_quant(const void* x, int in_dtype, int64_t numel, int out_dtype,
+                                   int round_mode, void* out, float* amax_out, float* scale_out,
+                                   void* workspace, size_t workspace_bytes, dt_stream_t stream);
+
+/* As above with two outputs from one read of x for the cast: e4m3fn with scale 448/amax and
+ * e5m2 with scale 57344/amax.  scale_out, if given, receives {scale_e4m3fn, scale_e5m2}.
+ * No counterpart in the reference (one dtype per call there).                             */
+DT_API int dt_dynamic_scaled_quant_pair(const void* x, int in_dtype, int64_t numel, int round_mode,
+                                        void* out_e4m3fn, void* out_e5m2, float* amax_out,
+                                        float* scale_out, void* workspace, size_t workspace_bytes,
+                                        dt_stream_t stream);
+
+/* The two stages of dt_dynamic_scaled_quant_pair as separate calls, for callers that keep the
+ * scales (delayed scaling: the reference's own flow is tensor_to_scale followed by
+ * saturated_cast, test/test_sat_cast.py:35-38) or time the stages separately.
+ * dt_amax_scales: amax_out[0] = max|x|, scale_out = {f32(448/max(amax,1e-12)),
+ * f32(57344/max(amax,1e-12))}; either may be NULL, the scales are also left in the workspace.
+ * dt_saturated_cast_pair: `scale` is that device pair; out_e4m3fn uses scale[0], out_e5m2
+ * scale[1].                                                                               */
+DT_API int dt_amax_scales(const void* x, int in_dtype, int64_t numel, float* amax_out, float* scale_out,
+                          void* workspace, size_t workspace_bytes, dt_stream_t stream);
+DT_API int dt_saturated_cast_pair(const void* x, int in_dtype, int64_t numel, const float* scale,
+                                  int round_mode, void* out_e4m3fn, void* out_e5m2, dt_stream_t stream);
+
+/* Row-wise: one amax / scale per row of a row-major [rows, cols] matrix, product in fp32
+ * (a [rows,1] scale promotes in eager).  amax_out / scale_out: fp32 [rows] or NULL.  No
+ * counterpart in the reference; the formulation is test/test_dynamic_quant.py:8-25 with
+ * amax(dim=-1, keepdim=True).                                                             */
+DT_API int dt_dynamic_scaled_quant_rowwise(const void* x, int in_dtype, int64_t rows, int64_t cols,
+                                           int out_dtype, void* out, float* amax_out,
+                                           float* scale_out, dt_stream_t stream);
+
+/* -------------------------------------------------------------- mx_fp8_quantize ------
+ * MXFP8 cast of a row-major [rows, cols] matrix: one E8M0 byte per 32 elements,
+ * byte = clamp(ceil(log2(blockmax)) - P + 127, 0, 254) with P = 8 (e4m3fn) or 15 (e5m2),
+ * payload = fp8_rne(clamp(x * 2^(127-byte))).  Replaces driss_torch::mx_fp8_quantize,
+ * src/mx_cast.cu:168-246 (host), :96-161 (kernel), :44-86 (exponent math).
+ *   axis 1: blocks along a row (the only mode of the reference); cols % 32 == 0
+ *   axis 0: blocks down a column; rows % 32 == 0
+ *   transpose 0: data [rows, cols]; scale [rows, cols/32] (axis 1) or [rows/32, cols] (axis 0)
+ *   transpose 1: data [cols, rows]; scale [cols/32, rows] (axis 1) or [cols, rows/32] (axis 0)
+ *                so (axis 0, transpose 1) equals the axis-1 cast of x^T.
+ * scale_layout DT_SCALE_BLOCKED writes the scale matrix directly in the layout
+ * dt_mx_fp8_bf16 reads (dt_blocked_scale_bytes(scale_rows, scale_cols) bytes, padding
+ * zeroed); it needs the scale matrix to be [outer, inner/32], i.e. (axis 1, transpose 0)
+ * or (axis 0, transpose 1).  x must be 16-byte aligned; in_dtype F32, BF16 or F16.        */
+DT_API int dt_mx_fp8_quantize(const void* x, int in_dtype, int64_t rows, int64_t cols, int axis,
+                              int transpose, int out_dtype, int scale_layout, void* data,
+                              uint8_t* scale, dt_stream_t stream);
+
+/* bytes of an [R, C] scale matrix in the blocked layout: 128*ceil(R/128) * 4*ceil(C/4) */
+DT_API int64_t dt_blocked_scale_bytes(int64_t R, int64_t C);
+
+/* plain [R, C] -> blocked (zero padded).  Stands in for transformer_nuggets' to_blocked,
+ * which the reference's test applies between the cast and the GEMM, test/test_mx.py:31-32 */
+DT_API int dt_to_blocked(const uint8_t* scale, int64_t R, int64_t C, uint8_t* out, dt_stream_t stream);
+
+/* ------------------------------------------------------------------ mx_fp8_bf16 ------
+ * out[M,N] (bf16, row stride ldo elements) = (A * 2^(sfa-127)) (B * 2^(sfb-127)), fp32
+ * accumulation.  Replaces driss_torch::mx_fp8_bf16, src/mx_fp8_bf16.cu:217-241 (host),
+ * :168-214 (operand contract), :36-163 (GEMM).  a: e4m3fn [M,K], row stride lda bytes;
+ * b: the reference's [K,N] tensor with stride(0)==1, i.e. e4m3fn [N,K] with row stride ldb
+ * bytes; sfa / sfb: E8M0 in the blocked layout, dt_blocked_scale_bytes(M, K/32) and
+ * (N, K/32) bytes.  K % 128 == 0, lda % 16 == 0, ldb % 16 == 0, a, b 16-byte aligned
+ * (:190-195), out 8-byte aligned, N % 4 == 0 and ldo % 4 == 0 (the reference asks N % 8, :187).                                     */
+DT_API int dt_mx_fp8_bf16(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb,
+                          int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, void* out,
+                          int64_t ldo, dt_stream_t stream);
+
+/* ---------------------------------------------------------------- tuning -------------
+ * Launch-shape knobs for benchmarking sweeps ("amax.blocks_per_cu", ...).  Returns DT_OK
+ * or DT_ERR_INVALID_MODE for an unknown key.  Not part of the reference's surface.        */
+DT_API int dt_set_tuning(const char* key, int value);
+DT_API int dt_get_tuning(const char* key, int* value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DRISS_TORCH_HIP_H */

@@ -1,0 +1,251 @@
+"""GPU parity: mx_fp8_quantize (all orientations and scale layouts) bit for bit against the CPU
+oracle, and mx_fp8_bf16 against the dequantized matmul, on the reference's shape lists
+(test/test_mx.py:42-59,70-84) and the benchmark configs."""
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from oracle import eager
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+
+
+@pytest.fixture(scope="module")
+def d(gpu_device):
+    import driss_torch_amd
+
+    return driss_torch_amd
+
+
+@pytest.fixture(scope="module")
+def cabi(gpu_device):
+    from driss_torch_amd import cabi as c
+
+    return c
+
+
+# --------------------------------------------------------------------------- MX cast
+@pytest.mark.parametrize("size", [(128, 32), (256, 32), (8192, 32), (128, 64), (128, 128), (128, 8192), (256, 64),
+                                  (256, 128), (8192, 8192)], ids=lambda s: f"{s[0]}x{s[1]}")
+def test_mx_cast_reference_shapes(d, size):
+    """test/test_mx.py:70-94: positive uniform bf16 input, data and scale bit exact"""
+    a = util.uniform(size, 400 + size[0] + size[1])
+    data, scale = d.mx_fp8_quantize(a.cuda())
+    assert data.dtype == E4 and data.shape == a.shape
+    assert scale.dtype == torch.float8_e8m0fnu and scale.shape == (size[0] * size[1] // 32,)
+    rd, rs = co.mx_quantize(a)
+    assert torch.equal(util.codes(scale), rs.flatten())
+    assert torch.equal(util.codes(data), rd)
+    if size[0] * size[1] <= 1 << 20:
+        es, ed = eager.to_mx(a, E4)
+        assert torch.equal(util.codes(scale), es.flatten()) and torch.equal(util.codes(data), util.codes(ed))
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("out_dtype", [E4, E5])
+@pytest.mark.parametrize("axis,transpose", [(1, False), (0, False), (0, True), (1, True)])
+@pytest.mark.parametrize("shape", [(32, 32), (96, 160), (160, 96), (512, 1056), (1056, 512)])
+def test_mx_cast_orientations(d, in_dtype, out_dtype, axis, transpose, shape):
+    a = util.student_t(shape, 500 + shape[0], in_dtype)
+    a[0, 0] = 0.0
+    a[-1, -1] = -0.0
+    if in_dtype != torch.float16:
+        a[3, 5] = 3e38 if in_dtype == torch.float32 else 3e38
+    data, scale = d.mx_fp8_quantize(a.cuda(), 32, axis, transpose, out_dtype)
+    rd, rs = co.mx_quantize(a, axis=axis, transpose=transpose, out_dtype=out_dtype)
+    assert data.shape == rd.shape and scale.numel() == rs.numel()
+    assert torch.equal(util.codes(scale), rs.flatten())
+    assert torch.equal(util.codes(data), rd)
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("axis,transpose", [(1, False), (0, False), (0, True)])
+def test_mx_cast_special_blocks(d, in_dtype, axis, transpose):
+    a = util.student_t((64, 128), 61, in_dtype)
+    a[0:32, 0:32] = 0                      # all-zero blocks in either direction -> byte 0, zero payload
+    a[40, 70] = float("nan")               # NaN block -> byte 255, NaN payload
+    a[33, 33] = float("inf")               # inf saturates, byte from exponent 128
+    tiny = 1e-40 if in_dtype == torch.float32 else (2.0 ** -133 if in_dtype == torch.bfloat16 else 2.0 ** -24)
+    a[32:64, 96:128] = tiny                # subnormal maxima
+    a[:, 100] = torch.where(torch.arange(64) % 2 == 0, 1.0, -1.0).to(in_dtype) * tiny
+    data, scale = d.mx_fp8_quantize(a.cuda(), 32, axis, transpose, E4)
+    rd, rs = co.mx_quantize(a, axis=axis, transpose=transpose)
+    assert torch.equal(util.codes(scale), rs.flatten())
+    assert torch.equal(util.codes(data), rd)
+
+
+def test_mx_cast_blocked_scales_and_errors(d, cabi):
+    for shape, axis in [((256, 512), 1), ((129, 160), 1), ((512, 256), 0), ((160, 129 * 1), 0), ((96, 200), 0)]:
+        a = util.student_t(shape, 71 + shape[0])
+        data, scale = d.mx_fp8_quantize_blocked(a.cuda(), axis=axis)
+        rd, rs = co.mx_quantize(a, axis=axis, transpose=(axis == 0))
+        assert torch.equal(util.codes(data), rd)
+        assert torch.equal(util.codes(scale), co.to_blocked(rs))
+        # to_blocked on its own
+        assert torch.equal(d.to_blocked(rs.cuda()).cpu(), eager.to_blocked(rs))
+    x = util.student_t((64, 48), 72).cuda()
+    with pytest.raises(RuntimeError):
+        d.mx_fp8_quantize(x)  # 48 % 32 != 0 (src/mx_cast.cu:218-219)
+    with pytest.raises(RuntimeError):
+        d.mx_fp8_quantize(x.t())  # not contiguous
+    with pytest.raises(RuntimeError):
+        d.mx_fp8_quantize(x.double())
+    with pytest.raises(RuntimeError):
+        d.mx_fp8_quantize(x, 16)
+    with pytest.raises(RuntimeError):
+        d.mx_fp8_quantize(x, 32, 1, False, torch.bfloat16)
+    assert d.mx_fp8_quantize(x, 32, 0)[0].shape == (64, 48)
+
+
+def test_mx_cast_config4_full_size(d):
+    a = util.student_t((8192, 8192), 1004)
+    ag = a.cuda()
+    data, scale = d.mx_fp8_quantize(ag)
+    rd, rs = co.mx_quantize(a)
+    assert torch.equal(util.codes(scale), rs.flatten()) and torch.equal(util.codes(data), rd)
+    # column-wise blocks, output transposed == row-wise cast of x^T (checked against both)
+    dT, sT = d.mx_fp8_quantize(ag, 32, 0, True)
+    rdT, rsT = co.mx_quantize(a, axis=0, transpose=True)
+    assert torch.equal(util.codes(sT), rsT.flatten()) and torch.equal(util.codes(dT), rdT)
+    d2, s2 = d.mx_fp8_quantize(ag.t().contiguous())
+    assert torch.equal(util.codes(d2), util.codes(dT)) and torch.equal(util.codes(s2), util.codes(sT))
+    # column-wise blocks in place
+    d0, s0 = d.mx_fp8_quantize(ag, 32, 0, False)
+    assert torch.equal(util.codes(d0), rdT.t()) and torch.equal(util.codes(s0).view(256, 8192), rsT.t())
+    # round trip: dequantized value within 2^-4 of the block maximum
+    deq = eager.mx_dequant(data.cpu()[:256], rs[:256])
+    x = a[:256].float().reshape(256, 256, 32)
+    assert ((deq.reshape(256, 256, 32) - x).abs().amax(-1) <= x.abs().amax(-1) * 2**-4).all()
+
+
+# --------------------------------------------------------------------------- MX GEMM
+def _operands(d, M, K, N, seed, dist="rand"):
+    mk = util.uniform if dist == "rand" else util.normal
+    a = mk((M, K), seed).cuda()
+    b = mk((N, K), seed + 1).cuda()
+    a_data, a_scale = d.mx_fp8_quantize(a)
+    b_data, b_scale = d.mx_fp8_quantize(b)
+    a_sc = a_scale.view(M, K // 32)
+    b_sc = b_scale.view(N, K // 32)
+    return a_data, a_sc, b_data, b_sc
+
+
+def _check_gemm(d, M, K, N, seed, dist):
+    a_data, a_sc, b_data, b_sc = _operands(d, M, K, N, seed, dist)
+    out = d.mx_fp8_bf16(a_data, b_data.t(), d.to_blocked(a_sc), d.to_blocked(b_sc))
+    assert out.shape == (M, N) and out.dtype == torch.bfloat16
+    ad, asc, bd, bsc = a_data.cpu(), util.codes(a_sc), b_data.cpu(), util.codes(b_sc)
+    da, db = eager.mx_dequant(ad, asc), eager.mx_dequant(bd, bsc)
+    ref = da.double() @ db.double().T
+    got = out.cpu().double()
+    sqnr = eager.compute_error(ref, got).item()
+    # Tolerance.  The only rounding besides fp32 accumulation is the final bf16 store (relative
+    # 2^-9); measured against sum_k |a||b| that bounds every entry, and gives an SQNR well
+    # above 45 dB even for zero-mean data.  The reference's bar is SQNR > 80 dB against a
+    # *bf16* matmul of the same operands on rand data (test/test_mx.py:64); against the exact
+    # product a bf16 output cannot exceed ~57 dB, so the bar here is 50 dB plus the entrywise
+    # bound.
+    bound = da.abs().double() @ db.abs().double().T
+    err = (got - ref).abs()
+    assert (err <= bound * 2**-8 + 1e-30).all(), f"max rel {(err / bound).max().item():.3e}"
+    assert sqnr > 50, sqnr
+    return out, ref
+
+
+@pytest.mark.parametrize("size", [(128, 128, 128), (256, 256, 256), (384, 384, 384), (512, 512, 512), (768, 768, 768),
+                                  (1024, 1024, 1024), (128, 256, 384), (256, 384, 512), (129, 256, 384), (133, 512, 528)],
+                         ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+@pytest.mark.parametrize("dist", ["rand", "randn"])
+def test_mx_gemm_reference_sizes(d, size, dist):
+    M, K, N = size
+    _check_gemm(d, M, K, N, 600 + M + N, dist)
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("size", [(128, 128, 128), (512, 256, 640), (133, 512, 528), (300, 1024, 264)])
+def test_mx_gemm_both_tile_shapes(d, cabi, variant, size):
+    cabi.set_tuning("gemm.variant", variant)
+    try:
+        _check_gemm(d, *size, 700, "randn")
+    finally:
+        cabi.set_tuning("gemm.variant", 0)
+
+
+def test_mx_gemm_small_vs_c_oracle_exact_products(d):
+    """with power-of-two operands every product and partial sum is exact, so the bf16 result
+    must equal the C oracle's float64 reference rounded to bf16, bit for bit"""
+    M, K, N = 160, 256, 136
+    g = util.gen(81)
+    a = torch.exp2(torch.randint(-6, 6, (M, K), generator=g).float()) * torch.where(torch.rand(M, K, generator=g) < 0.5, -1.0, 1.0)
+    b = torch.exp2(torch.randint(-6, 6, (N, K), generator=g).float()) * torch.where(torch.rand(N, K, generator=g) < 0.5, -1.0, 1.0)
+    # sparse so that sums stay within bf16's 8 significant bits
+    a = a * (torch.rand(M, K, generator=g) < 0.02)
+    b = b * (torch.rand(N, K, generator=g) < 0.5)
+    ad, asc = d.mx_fp8_quantize(a.bfloat16().cuda())
+    bd, bsc = d.mx_fp8_quantize(b.bfloat16().cuda())
+    out = d.mx_fp8_bf16(ad, bd.t(), d.to_blocked(asc.view(M, K // 32)), d.to_blocked(bsc.view(N, K // 32)))
+    ref = co.mx_gemm_ref(util.codes(ad), util.codes(bd), co.to_blocked(util.codes(asc).view(M, K // 32)),
+                         co.to_blocked(util.codes(bsc).view(N, K // 32)))
+    assert torch.equal(out.cpu(), ref.bfloat16())
+
+
+def test_mx_gemm_scale_bytes_are_applied_per_row_and_kblock(d):
+    M, K, N = 256, 512, 256
+    a_data, a_sc, b_data, b_sc = _operands(d, M, K, N, 83, "randn")
+    base = d.mx_fp8_bf16(a_data, b_data.t(), d.to_blocked(a_sc), d.to_blocked(b_sc)).float()
+    sc2 = util.codes(a_sc).clone()
+    sc2[77, :] += 3  # scale row 77 of A by 8
+    out = d.mx_fp8_bf16(a_data, b_data.t(), d.to_blocked(sc2.cuda()), d.to_blocked(b_sc)).float()
+    assert torch.equal(out[77], base[77] * 8)
+    assert torch.equal(out[:77], base[:77]) and torch.equal(out[78:], base[78:])
+    # zero all but one K-block of B: result equals the partial product of that block
+    kb = 5
+    b2 = util.codes(b_data).clone()
+    mask = torch.zeros(K, dtype=torch.bool)
+    mask[kb * 32:(kb + 1) * 32] = True
+    b2[:, ~mask] = 0
+    out = d.mx_fp8_bf16(a_data, b2.view(torch.float8_e4m3fn).cuda().t(), d.to_blocked(a_sc), d.to_blocked(b_sc))
+    da = eager.mx_dequant(a_data.cpu(), util.codes(a_sc))[:, mask]
+    db = eager.mx_dequant(b_data.cpu(), util.codes(b_sc))[:, mask]
+    ref = (da.double() @ db.double().T)
+    assert ((out.cpu().double() - ref).abs() <= ref.abs() * 2**-8 + 1e-6).all()
+
+
+def test_mx_gemm_argument_errors(d):
+    M, K, N = 128, 128, 128
+    a_data, a_sc, b_data, b_sc = _operands(d, M, K, N, 85)
+    sa, sb = d.to_blocked(a_sc), d.to_blocked(b_sc)
+    with pytest.raises(RuntimeError):
+        d.mx_fp8_bf16(a_data, b_data, sa, sb)  # b not K-contiguous (src/mx_fp8_bf16.cu:211-213)
+    with pytest.raises(RuntimeError):
+        d.mx_fp8_bf16(a_data, b_data.t(), sa[:-1], sb)  # scale length (src/mx_fp8_bf16.cu:197-205)
+    with pytest.raises(RuntimeError):
+        d.mx_fp8_bf16(a_data[:, :64], b_data.t(), sa, sb)  # K mismatch
+    with pytest.raises(RuntimeError):
+        d.mx_fp8_bf16(a_data.view(torch.uint8), b_data.t(), sa, sb)
+    with pytest.raises(RuntimeError):
+        d.mx_fp4_bf16(a_data, b_data.t(), sa, sb)
+
+
+def test_mx_gemm_config5_full_size(d):
+    """8192^3 from the row-wise cast of N(0,1) operands, scales written blocked by the cast
+    itself; checked on sampled rows against the float64 dequantized product."""
+    M = N = K = 8192
+    a = util.normal((M, K), 1005).cuda()
+    b = util.normal((N, K), 1006).cuda()
+    a_data, sa = d.mx_fp8_quantize_blocked(a)
+    b_data, sb = d.mx_fp8_quantize_blocked(b)
+    out = d.mx_fp8_bf16(a_data, b_data.t(), sa, sb)
+    _, a_plain = d.mx_fp8_quantize(a)
+    _, b_plain = d.mx_fp8_quantize(b)
+    rows = torch.tensor([0, 1, 127, 128, 4095, 4096, 5000, 8191])
+    da = eager.mx_dequant(a_data[rows.cuda()].cpu(), util.codes(a_plain).view(M, K // 32)[rows])
+    db = eager.mx_dequant(b_data.cpu(), util.codes(b_plain).view(N, K // 32))
+    ref = da.double() @ db.double().T
+    got = out[rows.cuda()].cpu().double()
+    bound = da.abs().double() @ db.abs().double().T
+    assert ((got - ref).abs() <= bound * 2**-8).all()
+    assert eager.compute_error(ref, got).item() > 50
