@@ -1,9 +1,11 @@
 // dt_mx_fp8_bf16: block-scaled e4m3 x e4m3 -> bf16 GEMM on the CDNA4 scaled MFMA (C ABI).
 //
 // D[M,N] = sum_k (A[m,k] 2^(sfa[m,k/32]-127)) (B[n,k] 2^(sfb[n,k/32]-127)); A is [M,K] and B is
-// [N,K], both with K contiguous, so every MFMA operand fragment is a run of 32 consecutive
-// bytes of one row.  v_mfma_scale_f32_16x16x128_f8f6f4 applies one E8M0 byte per lane to the
-// 32 values that lane supplies, which is exactly one MX block.
+// [N,K], both with K contiguous.  Operand layout of v_mfma_scale_f32_16x16x128_f8f6f4 (measured
+// on gfx950): lane l = 16*g + i supplies, for row i, K = 16g..16g+15 in its first four VGPRs
+// and K = 64+16g..64+16g+15 in the last four; the E8M0 byte lane l supplies scales K-block g
+// (K = 32g..32g+31) of row i.  So a fragment is two 16-byte reads 64 bytes apart, and one MX
+// block maps to one scale lane.
 //
 // A workgroup of 4 waves owns a BM x BN output tile and walks K in steps of 128.  The A and B
 // panels of a step are staged through LDS (rows padded by 16 bytes so the 16-byte fragment
@@ -134,14 +136,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     v8i fa[TM], fb[TN];
 #pragma unroll
     for (int t = 0; t < TM; ++t) {
-      const uint8_t* p = ldsA + (wm * WM + t * 16 + l16) * kLdsRow + kq * 32;
-      const u32x4 lo = *reinterpret_cast<const u32x4*>(p), hi = *reinterpret_cast<const u32x4*>(p + 16);
+      const uint8_t* p = ldsA + (wm * WM + t * 16 + l16) * kLdsRow + kq * 16;
+      const u32x4 lo = *reinterpret_cast<const u32x4*>(p), hi = *reinterpret_cast<const u32x4*>(p + 64);
       fa[t] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
     }
 #pragma unroll
     for (int t = 0; t < TN; ++t) {
-      const uint8_t* p = ldsB + (wn * WN + t * 16 + l16) * kLdsRow + kq * 32;
-      const u32x4 lo = *reinterpret_cast<const u32x4*>(p), hi = *reinterpret_cast<const u32x4*>(p + 16);
+      const uint8_t* p = ldsB + (wn * WN + t * 16 + l16) * kLdsRow + kq * 16;
+      const u32x4 lo = *reinterpret_cast<const u32x4*>(p), hi = *reinterpret_cast<const u32x4*>(p + 64);
       fb[t] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
     }
 #pragma unroll

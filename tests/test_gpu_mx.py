@@ -175,12 +175,14 @@ def test_mx_gemm_both_tile_shapes(d, cabi, variant, size):
 
 
 def test_mx_gemm_small_vs_c_oracle_exact_products(d):
-    """with power-of-two operands every product and partial sum is exact, so the bf16 result
-    must equal the C oracle's float64 reference rounded to bf16, bit for bit"""
+    """with power-of-two operands in a narrow exponent range every product and partial sum is
+    exact, so the bf16 result must equal the C oracle's float64 reference rounded to bf16, bit
+    for bit.  (Over a 2^22 range the MFMA's internal alignment drops the smallest addends --
+    measured: 2 of 21760 entries lose a 2^-12 term next to 2^10 ones -- hence the range here.)"""
     M, K, N = 160, 256, 136
     g = util.gen(81)
-    a = torch.exp2(torch.randint(-6, 6, (M, K), generator=g).float()) * torch.where(torch.rand(M, K, generator=g) < 0.5, -1.0, 1.0)
-    b = torch.exp2(torch.randint(-6, 6, (N, K), generator=g).float()) * torch.where(torch.rand(N, K, generator=g) < 0.5, -1.0, 1.0)
+    a = torch.exp2(torch.randint(-3, 3, (M, K), generator=g).float()) * torch.where(torch.rand(M, K, generator=g) < 0.5, -1.0, 1.0)
+    b = torch.exp2(torch.randint(-3, 3, (N, K), generator=g).float()) * torch.where(torch.rand(N, K, generator=g) < 0.5, -1.0, 1.0)
     # sparse so that sums stay within bf16's 8 significant bits
     a = a * (torch.rand(M, K, generator=g) < 0.02)
     b = b * (torch.rand(N, K, generator=g) < 0.5)
@@ -211,7 +213,8 @@ def test_mx_gemm_scale_bytes_are_applied_per_row_and_kblock(d):
     da = eager.mx_dequant(a_data.cpu(), util.codes(a_sc))[:, mask]
     db = eager.mx_dequant(b_data.cpu(), util.codes(b_sc))[:, mask]
     ref = (da.double() @ db.double().T)
-    assert ((out.cpu().double() - ref).abs() <= ref.abs() * 2**-8 + 1e-6).all()
+    bound = da.abs().double() @ db.abs().double().T
+    assert ((out.cpu().double() - ref).abs() <= bound * 2**-8).all()
 
 
 def test_mx_gemm_argument_errors(d):
