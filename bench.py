@@ -1,0 +1,270 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 / MX quantization path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
+
+A step is one pass of the per-tensor dynamic quantization over one 8192 x 8192 bf16 tensor
+(amax -> scales -> e4m3fn and e5m2 casts; two kernels, reached through the C ABI exactly as
+dt_dynamic_scaled_quant_pair issues them).  Inputs are resident in HBM before the timed
+region; steps rotate over enough buffer sets that no step finds its input in the 256 MB
+memory-side cache.  One JSON line is printed: the step throughput in algorithmic GB/s,
+the roofline figures of the dominant kernel (timed with events on the launch stream inside
+the same timed region), a table of every other kernel of the path (`kernels`), and the
+eager CPU formulation timed on this host's cores (`cpu_baseline`).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+FP8_PEAK_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
+MALL_BYTES = 256 << 20
+
+
+def _events(n):
+    import torch
+
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def time_launches(fn, nsets, steps, warmup):
+    """Average device time of fn(set_index) in microseconds: events around `steps` launches."""
+    import torch
+
+    for i in range(warmup):
+        fn(i % nsets)
+    torch.cuda.synchronize()
+    start, end = _events(2)
+    start.record()
+    for i in range(steps):
+        fn(i % nsets)
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) * 1e3 / steps
+
+
+def nsets_for(bytes_per_set):
+    """buffer sets needed so a set is evicted from the memory-side cache before it is reused"""
+    return max(2, -(-2 * MALL_BYTES // bytes_per_set) + 1)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-extra", action="store_true", help="skip the per-kernel table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every op of this path is a single-device kernel "
+              "(sharding is by rows with at most a 4-byte max-reduce); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from driss_torch_amd import cabi
+    from tests import util
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    K, W = args.steps, args.warmup
+
+    # ------------------------------------------------------------ headline step: config 2
+    R = C = 8192
+    numel = R * C
+    step_bytes = numel * (2 + 2 + 1 + 1)          # two reads of x, two fp8 writes
+    cast_bytes = numel * (2 + 1 + 1)              # dominant kernel: one read, two writes
+    amax_bytes = numel * 2
+    ns = nsets_for(numel * 4)
+    x_cpu = util.normal_with_outliers((R, C), 1002)
+    xs = [x_cpu.to(dev) if i == 0 else torch.roll(x_cpu, i, 0).to(dev) for i in range(ns)]
+    o4 = [torch.empty((R, C), dtype=torch.float8_e4m3fn, device=dev) for _ in range(ns)]
+    o5 = [torch.empty((R, C), dtype=torch.float8_e5m2, device=dev) for _ in range(ns)]
+    amax_out = torch.empty(1, dtype=torch.float32, device=dev)
+    scale_out = torch.empty(2, dtype=torch.float32, device=dev)
+    mode = cabi.ROUND_BF16_SCALE_PRODUCT
+
+    def step(i, ev=None):
+        s = i % ns
+        if ev:
+            ev[0].record()
+        cabi.amax_scales(xs[s], amax_out, scale_out)
+        if ev:
+            ev[1].record()
+        cabi.saturated_cast_pair(xs[s], scale_out, mode, o4[s], o5[s])
+        if ev:
+            ev[2].record()
+
+    for i in range(W):
+        step(i)
+    torch.cuda.synchronize()
+    evs = [_events(3) for _ in range(K)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        step(i, evs[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / K
+    amax_us = statistics.fmean(e[0].elapsed_time(e[1]) for e in evs) * 1e3
+    cast_us = statistics.fmean(e[1].elapsed_time(e[2]) for e in evs) * 1e3
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    cast_gbs = cast_bytes / (cast_us * 1e-6) / 1e9
+
+    result = {
+        "metric": "cast/amax HBM GB/s (% of 8 TB/s) at 8192^2 bf16; MXFP8 GEMM TFLOPS",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16->fp8 (fp32 arithmetic)",
+        "data": "synthetic",
+        "config": {"workload": "config 2: amax + dynamic_scaled_quant per tensor, bf16 [8192,8192] N(0,1) with 0.1% x100 "
+                               "outliers -> fp32 amax, scales, e4m3fn and e5m2 (402.7 MB algorithmic per step)",
+                   "buffer_sets": ns, "product_rounding": "bf16 product, bf16-rounded scale (eager with a 0-dim scale)"},
+        "roofline": {"kernel": "cast_kernel<bf16,e4m3fn+e5m2 pair>", "bound": "hbm", "achieved": round(cast_gbs, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(cast_gbs / HBM_PEAK_GBS, 4),
+                     "avg_launch_us": round(cast_us, 2), "algorithmic_bytes_per_launch": cast_bytes, "traffic": None},
+        "step_kernels_us": {"amax_kernel(+scales)": round(amax_us, 2), "cast_kernel(pair)": round(cast_us, 2),
+                            "amax_GBs": round(amax_bytes / (amax_us * 1e-6) / 1e9, 1)},
+    }
+    del xs, o4, o5
+    torch.cuda.empty_cache()
+
+    if not args.no_extra:
+        result["kernels"] = extra_kernels(torch, cabi, util, dev, K, W)
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch, x_cpu, step_bytes)
+    print(json.dumps(result))
+
+
+def extra_kernels(torch, cabi, util, dev, K, W):
+    """Every other kernel of the path at its benchmark config: rotated (HBM) and hot-cache."""
+    rows = []
+
+    def hbm_row(name, workload, nbytes, make_set, run):
+        one = make_set(0)
+        set_bytes = sum(t.numel() * t.element_size() for t in one if isinstance(t, torch.Tensor))
+        ns = nsets_for(set_bytes)
+        sets = [one] + [make_set(i) for i in range(1, ns)]
+        us = time_launches(lambda i: run(*sets[i]), ns, K, W)
+        us_hot = time_launches(lambda i: run(*sets[0]), 1, K, W)
+        gbs = nbytes / (us * 1e-6) / 1e9
+        rows.append({"kernel": name, "workload": workload, "bound": "hbm", "avg_us": round(us, 2),
+                     "achieved_GBs": round(gbs, 1), "frac_of_8TBs": round(gbs / HBM_PEAK_GBS, 4),
+                     "hot_cache_us": round(us_hot, 2), "hot_cache_GBs": round(nbytes / (us_hot * 1e-6) / 1e9, 1),
+                     "algorithmic_bytes": nbytes, "buffer_sets": ns})
+        del sets
+        torch.cuda.empty_cache()
+
+    bf16, f32 = torch.bfloat16, torch.float32
+    e4, e5 = torch.float8_e4m3fn, torch.float8_e5m2
+    scale1 = torch.full((1,), 37.0, device=dev)
+
+    def rnd(shape, dtype, i):
+        g = torch.Generator(device=dev).manual_seed(77 + i)
+        return torch.randn(shape, generator=g, device=dev, dtype=torch.float32).to(dtype)
+
+    n = 8192 * 8192
+    hbm_row("amax", "bf16 [8192,8192]", n * 2, lambda i: (rnd((8192, 8192), bf16, i), torch.empty(1, device=dev)),
+            lambda x, o: cabi.amax(x, o))
+    hbm_row("amax", "fp32 [8192,8192]", n * 4, lambda i: (rnd((8192, 8192), f32, i), torch.empty(1, device=dev)),
+            lambda x, o: cabi.amax(x, o))
+    for od, nm in ((e4, "e4m3fn"), (e5, "e5m2")):
+        hbm_row("saturated_cast", f"bf16 [8192,8192] -> {nm}", n * 3,
+                lambda i, od=od: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=od, device=dev)),
+                lambda x, o, od=od: cabi.saturated_cast(x, scale1, od, cabi.ROUND_BF16_SCALE_PRODUCT, o))
+    n1 = 4096 * 4096
+    hbm_row("saturated_cast", "config 1: bf16 [4096,4096] -> e4m3fn", n1 * 3,
+            lambda i: (rnd((4096, 4096), bf16, i), torch.empty((4096, 4096), dtype=e4, device=dev)),
+            lambda x, o: cabi.saturated_cast(x, scale1, e4, cabi.ROUND_BF16_SCALE_PRODUCT, o))
+    hbm_row("saturated_cast", "fp32 [8192,8192] -> e4m3fn", n * 5,
+            lambda i: (rnd((8192, 8192), f32, i), torch.empty((8192, 8192), dtype=e4, device=dev)),
+            lambda x, o: cabi.saturated_cast(x, scale1, e4, cabi.ROUND_F32, o))
+    nr = 16384 * 4096
+    for dt_, nm, b in ((f32, "fp32", 4), (bf16, "bf16", 2)):
+        hbm_row("dynamic_scaled_quant_rowwise", f"config 3: {nm} [16384,4096] -> e4m3fn", nr * (b + 1) + 16384 * 8,
+                lambda i, dt_=dt_: (rnd((16384, 4096), dt_, i), torch.empty((16384, 4096), dtype=e4, device=dev),
+                                    torch.empty((16384, 1), device=dev), torch.empty((16384, 1), device=dev)),
+                lambda x, o, a, s: cabi.dynamic_scaled_quant_rowwise(x, e4, o, a, s))
+    mxb = n * 2 + n + n // 32
+    hbm_row("mx_fp8_quantize rows", "config 4: bf16 [8192,8192], blocks along rows", mxb,
+            lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
+                       torch.empty((8192, 256), dtype=torch.uint8, device=dev)),
+            lambda x, dd, s: cabi.mx_fp8_quantize(x, 1, False, e4, cabi.SCALE_PLAIN, dd, s))
+    hbm_row("mx_fp8_quantize cols (transposed out)", "config 4: bf16 [8192,8192], blocks down columns", mxb,
+            lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
+                       torch.empty((8192, 256), dtype=torch.uint8, device=dev)),
+            lambda x, dd, s: cabi.mx_fp8_quantize(x, 0, True, e4, cabi.SCALE_PLAIN, dd, s))
+    hbm_row("mx_fp8_quantize cols (in place)", "config 4: bf16 [8192,8192], blocks down columns", mxb,
+            lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
+                       torch.empty((256, 8192), dtype=torch.uint8, device=dev)),
+            lambda x, dd, s: cabi.mx_fp8_quantize(x, 0, False, e4, cabi.SCALE_PLAIN, dd, s))
+
+    # MXFP8 GEMM, config 5
+    M = N = Kd = 8192
+    a = rnd((M, Kd), bf16, 1)
+    b = rnd((N, Kd), bf16, 2)
+    a_data, sfa = cabi.mx_fp8_quantize(a, 1, False, e4, cabi.SCALE_BLOCKED)
+    b_data, sfb = cabi.mx_fp8_quantize(b, 1, False, e4, cabi.SCALE_BLOCKED)
+    out = torch.empty((M, N), dtype=bf16, device=dev)
+    del a, b
+    us = time_launches(lambda i: cabi.mx_fp8_bf16(a_data, b_data, sfa, sfb, out), 1, max(5, K // 5), max(2, W // 5))
+    flops = 2.0 * M * N * Kd
+    tf = flops / (us * 1e-6) / 1e12
+    rows.append({"kernel": "mx_fp8_bf16", "workload": "config 5: 8192^3 e4m3 x e4m3, E8M0 block-32 scales -> bf16",
+                 "bound": "mfma", "avg_us": round(us, 2), "achieved_TFLOPs": round(tf, 1),
+                 "frac_of_fp8_peak": round(tf / FP8_PEAK_TFLOPS, 4), "flops": flops})
+    return rows
+
+
+def cpu_baseline(torch, x_cpu, step_bytes):
+    """The eager formulation the reference's tests use, on this host's cores."""
+    from oracle import eager
+
+    cores = os.cpu_count() or 1
+    # worker pools are sized to the box's CPU share, whatever cpu_count says
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+
+    def once():
+        t0 = time.perf_counter()
+        for od in (torch.float8_e4m3fn, torch.float8_e5m2):
+            eager.dynamic_scaled_quant(x_cpu, od)
+        return time.perf_counter() - t0
+
+    once()
+    ts = [once() for _ in range(3)]
+    t = statistics.median(ts)
+    model = ""
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {"value": round(step_bytes / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "the whole config-2 tensor (bf16 8192x8192), eager amax -> scale -> cast for e4m3fn and e5m2, "
+                      "median of 3 after one warm-up",
+            "seconds": round(t, 3), "cpu": model}
+
+
+if __name__ == "__main__":
+    main()

@@ -15,11 +15,11 @@ struct Knob {
 };
 // Launch-shape knobs.  Workgroups per CU for the persistent grids, chosen on MI355X.
 Knob g_knobs[] = {
-    {"amax.blocks_per_cu", 8},
-    {"cast.blocks_per_cu", 8},
-    {"cast.nontemporal", 0},
-    {"dynamic.cooperative", 0},
-    {"mx.blocks_per_cu", 8},
+    {"amax.blocks_per_cu", 1},
+    {"amax.stream_before_cast", 0},
+    {"cast.blocks_per_cu", 2},
+    {"cast.pair_blocks_per_cu", 3},
+    {"mx.blocks_per_cu", 16},
     {"mx.col_rbw", 0},
     {"gemm.variant", 0},
 };

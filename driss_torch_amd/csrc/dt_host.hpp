@@ -12,10 +12,10 @@ namespace dt {
 // ---- workspace layout (see dt_workspace_bytes in the public header) -----------------
 constexpr int kMaxPartials = 8192;          // upper bound on the grid of a reduction kernel
 constexpr size_t kWsTicket = 0;             // u32 arrival counter, zero between launches
+constexpr size_t kWsRunning = 128;          // u32 running max of |x| bits, zero between launches
 constexpr size_t kWsAmax = 64;              // f32 amax of the last reduction
 constexpr size_t kWsScale = 68;             // f32 scale[2] derived from it
-constexpr size_t kWsPartials = 256;         // u32 partial maxima, one per workgroup
-constexpr size_t kWsBytes = kWsPartials + sizeof(uint32_t) * kMaxPartials;
+constexpr size_t kWsBytes = 4096;
 
 struct DeviceFacts {
   int cu_count;

@@ -121,7 +121,7 @@ __global__ __launch_bounds__(kBlock) void mx_row_kernel(const void* __restrict__
 #pragma unroll
     for (int c = 0; c < LPB; ++c) {
       const uint32_t vi = vbase + c * kWave;
-      w[c] = vi < nvec ? v[vi] : u32x4{0u, 0u, 0u, 0u};
+      w[c] = vi < nvec ? ld_stream(v + vi) : u32x4{0u, 0u, 0u, 0u};
     }
     uint32_t mybyte = 0;
 #pragma unroll
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(kBlock) void mx_row_kernel(const void* __restrict__
         if constexpr (IN == DT_F32) {
           uint32_t r = pack4_finite<OUT>(as_f32(w[c].x) * s.mult, as_f32(w[c].y) * s.mult, as_f32(w[c].z) * s.mult,
                                          as_f32(w[c].w) * s.mult);
-          reinterpret_cast<uint32_t*>(data)[vi] = s.nan ? 0x7F7F7F7Fu : r;
+          st_stream(reinterpret_cast<uint32_t*>(data) + vi, s.nan ? 0x7F7F7F7Fu : r);
         } else {
           float f[8];
           unpack8<IN>(w[c], f);
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(kBlock) void mx_row_kernel(const void* __restrict__
           r.x = pack4_finite<OUT>(f[0] * s.mult, f[1] * s.mult, f[2] * s.mult, f[3] * s.mult);
           r.y = pack4_finite<OUT>(f[4] * s.mult, f[5] * s.mult, f[6] * s.mult, f[7] * s.mult);
           if (s.nan) r = u32x2{0x7F7F7F7Fu, 0x7F7F7F7Fu};
-          reinterpret_cast<u32x2*>(data)[vi] = r;
+          st_stream(reinterpret_cast<u32x2*>(data) + vi, r);
         }
       }
     }
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(kBlock) void mx_col_kernel(const void* __restrict__
     const uint64_t vfirst = (uint64_t)rb * 32u * row_vecs + col0 / kV;
     u32x4 w[32];
 #pragma unroll
-    for (int i = 0; i < 32; ++i) w[i] = v[vfirst + (uint64_t)i * row_vecs];
+    for (int i = 0; i < 32; ++i) w[i] = ld_stream(v + vfirst + (uint64_t)i * row_vecs);
 
     // per-column magnitude maxima
     uint32_t cm[kV];
@@ -254,8 +254,8 @@ __global__ __launch_bounds__(kBlock) void mx_col_kernel(const void* __restrict__
                              (nanc[4 * q + 2] ? 0xFF0000u : 0u) | (nanc[4 * q + 3] ? 0xFF000000u : 0u);
           r[q] = (r[q] & ~nanmask) | (0x7F7F7F7Fu & nanmask);
         }
-        if constexpr (kW == 2) *reinterpret_cast<u32x2*>(drow + (uint64_t)i * cols) = u32x2{r[0], r[1]};
-        else *reinterpret_cast<uint32_t*>(drow + (uint64_t)i * cols) = r[0];
+        if constexpr (kW == 2) st_stream(reinterpret_cast<u32x2*>(drow + (uint64_t)i * cols), u32x2{r[0], r[1]});
+        else st_stream(reinterpret_cast<uint32_t*>(drow + (uint64_t)i * cols), r[0]);
       }
       // scales [rows/32, cols]: kV adjacent bytes
       uint8_t* srow = scale + (uint64_t)rb * cols + col0;
@@ -272,6 +272,7 @@ __global__ __launch_bounds__(kBlock) void mx_col_kernel(const void* __restrict__
           if (nanc[c]) r[q] = 0x7F7F7F7Fu;
         }
         u32x4* dcol = reinterpret_cast<u32x4*>(data + (uint64_t)(col0 + c) * rows + (uint64_t)rb * 32u);
+        // plain stores: neighbouring tiles complete these 128-byte lines in the L2
         dcol[0] = u32x4{r[0], r[1], r[2], r[3]};
         dcol[1] = u32x4{r[4], r[5], r[6], r[7]};
       }

@@ -50,16 +50,15 @@ __device__ __forceinline__ uint32_t absbits_of(const void* x, int64_t i) {
 
 // --------------------------------------------------------------------------- amax ----
 // Every workgroup reduces a grid-strided share of the vectors to one unsigned magnitude,
-// publishes it in the workspace and takes a ticket; the workgroup that draws the last
-// ticket reduces the partials, writes amax (and, when NSCALES > 0, the fp8 scales derived
-// from it) and re-arms the ticket for the next launch.
-template <int IN, int UNROLL, int NSCALES>
+// folds it into a running maximum in the workspace with one atomic and takes a ticket; the
+// workgroup that draws the last ticket writes amax (and, when NSCALES > 0, the fp8 scales
+// derived from it) and re-arms the workspace for the next launch.
+template <int IN, int UNROLL, int NSCALES, bool NT>
 __global__ __launch_bounds__(kBlock) void amax_kernel(const void* __restrict__ x, Split sp,
                                                       uint8_t* __restrict__ ws, float* __restrict__ amax_out,
                                                       float* __restrict__ scale_out, float fmax0, float fmax1) {
   constexpr int kB = InTraits<IN>::kBytes, kV = InTraits<IN>::kVec;
   __shared__ uint32_t lds[kBlock / kWave];
-  __shared__ uint32_t is_last;
   const int tid = threadIdx.x;
   const u32x4* v = reinterpret_cast<const u32x4*>(static_cast<const uint8_t*>(x) + sp.head * kB);
 
@@ -78,11 +77,11 @@ __global__ __launch_bounds__(kBlock) void amax_kernel(const void* __restrict__ x
   for (; i + (UNROLL - 1) * stride < sp.nvec; i += UNROLL * stride) {
     u32x4 w[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) w[u] = v[i + u * stride];
+    for (int u = 0; u < UNROLL; ++u) w[u] = ld_maybe_stream<NT>(v + i + u * stride);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) absorb(w[u]);
   }
-  for (; i < sp.nvec; i += stride) absorb(v[i]);
+  for (; i < sp.nvec; i += stride) absorb(ld_maybe_stream<NT>(v + i));
 
   uint32_t m;
   if constexpr (IN == DT_F32) {
@@ -97,38 +96,38 @@ __global__ __launch_bounds__(kBlock) void amax_kernel(const void* __restrict__ x
   }
   m = block_umax<kBlock / kWave>(m, lds);
 
+  // One relaxed device-scope atomic max per workgroup carries the partial; a second one on the
+  // ticket tells the last workgroup to arrive.  No fence is needed: the max is an atomic with
+  // return, so it has been performed at the device's coherence point before the ticket is
+  // taken, and ticket order is total.  (A release/acquire fence here costs a cache
+  // write-back/invalidate per workgroup, which serialises: measured 10x the streaming time.)
   uint32_t* ticket = reinterpret_cast<uint32_t*>(ws + kWsTicket);
-  uint32_t* partials = reinterpret_cast<uint32_t*>(ws + kWsPartials);
+  uint32_t* running = reinterpret_cast<uint32_t*>(ws + kWsRunning);
   if (tid == 0) {
-    __hip_atomic_store(&partials[blockIdx.x], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __threadfence();  // publish the partial before the ticket
-    uint32_t t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    is_last = (t == gridDim.x - 1) ? 1u : 0u;
-  }
-  __syncthreads();
-  if (!is_last) return;
-
-  __threadfence();
-  uint32_t r = 0;
-  for (int j = tid; j < (int)gridDim.x; j += kBlock)
-    r = umax(r, __hip_atomic_load(&partials[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-  r = block_umax<kBlock / kWave>(r, lds);
-  if (tid == 0) {
-    const float amax = as_f32(r);
-    *reinterpret_cast<float*>(ws + kWsAmax) = amax;
-    if (amax_out) *amax_out = amax;
-    if constexpr (NSCALES > 0) {
-      float* wscale = reinterpret_cast<float*>(ws + kWsScale);
-      const float s0 = amax_to_scale(amax, fmax0);
-      wscale[0] = s0;
-      if (scale_out) scale_out[0] = s0;
-      if constexpr (NSCALES > 1) {
-        const float s1 = amax_to_scale(amax, fmax1);
-        wscale[1] = s1;
-        if (scale_out) scale_out[1] = s1;
+    uint32_t before = __hip_atomic_fetch_max(running, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // make the ticket depend on the returned value so the two atomics cannot be reordered
+    uint32_t one = 1u;
+    asm volatile("v_and_or_b32 %0, %1, 0, %0" : "+v"(one) : "v"(before));
+    uint32_t t = __hip_atomic_fetch_add(ticket, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (t == gridDim.x - 1) {
+      // last to arrive: every other workgroup's max is already in `running`
+      const uint32_t r = __hip_atomic_exchange(running, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // re-arm
+      __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);                          // re-arm
+      const float amax = as_f32(r);
+      *reinterpret_cast<float*>(ws + kWsAmax) = amax;
+      if (amax_out) *amax_out = amax;
+      if constexpr (NSCALES > 0) {
+        float* wscale = reinterpret_cast<float*>(ws + kWsScale);
+        const float s0 = amax_to_scale(amax, fmax0);
+        wscale[0] = s0;
+        if (scale_out) scale_out[0] = s0;
+        if constexpr (NSCALES > 1) {
+          const float s1 = amax_to_scale(amax, fmax1);
+          wscale[1] = s1;
+          if (scale_out) scale_out[1] = s1;
+        }
       }
     }
-    __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // re-arm
   }
 }
 
@@ -140,7 +139,9 @@ inline int reduction_grid(int64_t nvec, int unroll, const char* knob) {
   return want < 1 ? 1 : (int)want;
 }
 
-// Enqueue the amax reduction.  nscales: 0 = amax only, 1 = scale for fmax0, 2 = both.
+// Enqueue the amax reduction.  nscales: 0 = amax only, 1 = scale for fmax0, 2 = both.  With
+// scales a cast pass over the same tensor follows, so the loads are left cacheable unless
+// the "amax.stream_before_cast" knob says otherwise.
 template <int IN>
 inline int launch_amax(const void* x, int64_t numel, void* ws, float* amax_out, float* scale_out, int nscales,
                        float fmax0, float fmax1, hipStream_t stream) {
@@ -148,12 +149,12 @@ inline int launch_amax(const void* x, int64_t numel, void* ws, float* amax_out, 
   Split sp = split_for_vectors<IN>(x, numel);
   int grid = reduction_grid(sp.nvec, kUnroll, "amax.blocks_per_cu");
   uint8_t* w = static_cast<uint8_t*>(ws);
-  if (nscales == 0)
-    amax_kernel<IN, kUnroll, 0><<<grid, kBlock, 0, stream>>>(x, sp, w, amax_out, scale_out, fmax0, fmax1);
-  else if (nscales == 1)
-    amax_kernel<IN, kUnroll, 1><<<grid, kBlock, 0, stream>>>(x, sp, w, amax_out, scale_out, fmax0, fmax1);
-  else
-    amax_kernel<IN, kUnroll, 2><<<grid, kBlock, 0, stream>>>(x, sp, w, amax_out, scale_out, fmax0, fmax1);
+  const bool nt = nscales == 0 || tuning("amax.stream_before_cast");
+#define DT_AMAX(NS, NT) amax_kernel<IN, kUnroll, NS, NT><<<grid, kBlock, 0, stream>>>(x, sp, w, amax_out, scale_out, fmax0, fmax1)
+  if (nscales == 0) DT_AMAX(0, true);
+  else if (nscales == 1) { if (nt) DT_AMAX(1, true); else DT_AMAX(1, false); }
+  else { if (nt) DT_AMAX(2, true); else DT_AMAX(2, false); }
+#undef DT_AMAX
   return launch_status();
 }
 
@@ -163,16 +164,25 @@ inline int launch_amax(const void* x, int64_t numel, void* ws, float* amax_out, 
 template <int IN, int OUT, bool ROUND_BF16>
 __device__ __forceinline__ void cast_vec(u32x4 w, float s, uint8_t* __restrict__ out, int64_t vec_index) {
   if constexpr (IN == DT_F32) {
-    uint32_t r = pack4<OUT>(scaled<false>(as_f32(w.x), s), scaled<false>(as_f32(w.y), s),
-                            scaled<false>(as_f32(w.z), s), scaled<false>(as_f32(w.w), s));
-    reinterpret_cast<uint32_t*>(out)[vec_index] = r;
+    const float p0 = as_f32(w.x) * s, p1 = as_f32(w.y) * s, p2 = as_f32(w.z) * s, p3 = as_f32(w.w) * s;
+    st_stream(reinterpret_cast<uint32_t*>(out) + vec_index, pack4<OUT>(p0, p1, p2, p3));
   } else {
+    float p[8] = {bf16_lo(w.x) * s, bf16_hi(w.x) * s, bf16_lo(w.y) * s, bf16_hi(w.y) * s,
+                  bf16_lo(w.z) * s, bf16_hi(w.z) * s, bf16_lo(w.w) * s, bf16_hi(w.w) * s};
+    if constexpr (ROUND_BF16) {
+      round2_to_bf16(p[0], p[1]); round2_to_bf16(p[2], p[3]);
+      round2_to_bf16(p[4], p[5]); round2_to_bf16(p[6], p[7]);
+    }
     u32x2 r;
-    r.x = pack4<OUT>(scaled<ROUND_BF16>(bf16_lo(w.x), s), scaled<ROUND_BF16>(bf16_hi(w.x), s),
-                     scaled<ROUND_BF16>(bf16_lo(w.y), s), scaled<ROUND_BF16>(bf16_hi(w.y), s));
-    r.y = pack4<OUT>(scaled<ROUND_BF16>(bf16_lo(w.z), s), scaled<ROUND_BF16>(bf16_hi(w.z), s),
-                     scaled<ROUND_BF16>(bf16_lo(w.w), s), scaled<ROUND_BF16>(bf16_hi(w.w), s));
-    reinterpret_cast<u32x2*>(out)[vec_index] = r;
+    r.x = pack4_clamped<OUT>(p[0], p[1], p[2], p[3]);
+    r.y = pack4_clamped<OUT>(p[4], p[5], p[6], p[7]);
+    const bool any_nan = (p[0] != p[0]) | (p[1] != p[1]) | (p[2] != p[2]) | (p[3] != p[3]) | (p[4] != p[4]) |
+                         (p[5] != p[5]) | (p[6] != p[6]) | (p[7] != p[7]);
+    if (__builtin_expect(any_nan, 0)) {
+      r.x = nan_patch4(r.x, p[0], p[1], p[2], p[3]);
+      r.y = nan_patch4(r.y, p[4], p[5], p[6], p[7]);
+    }
+    st_stream(reinterpret_cast<u32x2*>(out) + vec_index, r);
   }
 }
 
@@ -203,7 +213,7 @@ __global__ __launch_bounds__(kBlock) void cast_kernel(const void* __restrict__ x
   for (; i + (UNROLL - 1) * stride < nvec; i += UNROLL * stride) {
     u32x4 w[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) w[u] = v[i + u * stride];
+    for (int u = 0; u < UNROLL; ++u) w[u] = ld_stream(v + i + u * stride);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       cast_vec<IN, OUT, ROUND_BF16>(w[u], s, out, i + u * stride);
@@ -211,7 +221,7 @@ __global__ __launch_bounds__(kBlock) void cast_kernel(const void* __restrict__ x
     }
   }
   for (; i < nvec; i += stride) {
-    u32x4 w = v[i];
+    u32x4 w = ld_stream(v + i);
     cast_vec<IN, OUT, ROUND_BF16>(w, s, out, i);
     if constexpr (PAIR) cast_vec<IN, OUT2, ROUND_BF16>(w, s2, out2, i);
   }
@@ -240,14 +250,14 @@ __global__ __launch_bounds__(kBlock) void cast_kernel_unaligned(const void* __re
 template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR>
 inline int launch_cast_impl(const void* x, int64_t numel, const float* scale, void* out, void* out2,
                             hipStream_t stream) {
-  constexpr int kUnroll = 4;
+  constexpr int kUnroll = 8;
   constexpr size_t kStoreAlign = IN == DT_F32 ? 4 : 8;
   uint8_t* o = static_cast<uint8_t*>(out);
   uint8_t* o2 = static_cast<uint8_t*>(out2);
   const bool fast = aligned(x, 16) && aligned(out, kStoreAlign) && (!PAIR || aligned(out2, kStoreAlign));
   if (fast) {
     const int64_t nvec = numel / InTraits<IN>::kVec, tail = numel % InTraits<IN>::kVec;
-    int grid = reduction_grid(nvec, kUnroll, "cast.blocks_per_cu");
+    int grid = reduction_grid(nvec, kUnroll, PAIR ? "cast.pair_blocks_per_cu" : "cast.blocks_per_cu");
     cast_kernel<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR, kUnroll><<<grid, kBlock, 0, stream>>>(x, nvec, tail, scale, o, o2);
   } else {
     int grid = reduction_grid(numel, 1, "cast.blocks_per_cu");

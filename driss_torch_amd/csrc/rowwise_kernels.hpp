@@ -26,7 +26,7 @@ __global__ __launch_bounds__(kBlock) void rowwise_wave_kernel(const void* __rest
 #pragma unroll
   for (int u = 0; u < NV; ++u) {
     const int j = lane + u * kWave;
-    w[u] = j < row_vecs ? v[j] : u32x4{0u, 0u, 0u, 0u};
+    w[u] = j < row_vecs ? ld_stream(v + j) : u32x4{0u, 0u, 0u, 0u};
   }
   uint32_t m = 0;
 #pragma unroll
