@@ -46,7 +46,7 @@ __device__ __forceinline__ int64_t sf_group_offset(int r, int ks, int k_steps) {
   return ((int64_t)(r >> 7) * k_steps + ks) * 512 + (r & 31) * 16 + ((r & 127) >> 5) * 4;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST>
 __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const uint8_t* __restrict__ sfa,
     const uint8_t* __restrict__ sfb, int M, int N, int K, int64_t lda, int64_t ldb, uint16_t* __restrict__ out,
@@ -103,29 +103,36 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     gr = gr < N ? gr : N - 1;
     offB[i] = (uint32_t)((int64_t)gr * ldb + lchunk * 16);
   }
+  // Scales: one more wave-wide load per step.  256-row tiles: even waves bring the two A chunks
+  // (lanes 0-31 / 32-63), odd waves the two B chunks; 128-row tiles: lanes 0-31 bring the A
+  // chunk and lanes 32-63 the B chunk.  Every wave issues it (duplicates write identical bytes),
+  // which keeps the instruction stream free of branches.
   const int chunks_a = (M + 127) / 128, chunks_b = (N + 127) / 128;
-  int ca = m0 / 128 + (lane >> 5), cb = n0 / 128 + (lane >> 5);
-  ca = ca < chunks_a ? ca : chunks_a - 1;
-  cb = cb < chunks_b ? cb : chunks_b - 1;
-  const uint32_t offSA = (uint32_t)((int64_t)ca * k_steps * 512 + (lane & 31) * 16);
-  const uint32_t offSB = (uint32_t)((int64_t)cb * k_steps * 512 + (lane & 31) * 16);
-  auto fetch = [&](int ks, uint8_t* buf) {
-    const uint8_t* Ak = A + (int64_t)ks * kBK;
-    const uint8_t* Bk = B + (int64_t)ks * kBK;
-#pragma unroll
-    for (int i = 0; i < kLoadsA; ++i)
-      __builtin_amdgcn_global_load_lds((gptr_t)(Ak + offA[i]), (lptr_t)(buf + (wave * kLoadsA + i) * kGroupStride), 16, 0, 0);
-#pragma unroll
-    for (int i = 0; i < kLoadsB; ++i)
-      __builtin_amdgcn_global_load_lds((gptr_t)(Bk + offB[i]), (lptr_t)(buf + kOffB + (wave * kLoadsB + i) * kGroupStride),
-                                       16, 0, 0);
-    if (wave == 0) {
-      if (lane < 32 * (BM / 128))
-        __builtin_amdgcn_global_load_lds((gptr_t)(sfa + (int64_t)ks * 512 + offSA), (lptr_t)(buf + kOffSA), 16, 0, 0);
-    } else if (wave == 1) {
-      if (lane < 32 * (BN / 128))
-        __builtin_amdgcn_global_load_lds((gptr_t)(sfb + (int64_t)ks * 512 + offSB), (lptr_t)(buf + kOffSB), 16, 0, 0);
+  const bool lane_is_b = (BM == 256) ? (wave & 1) != 0 : lane >= 32;
+  int chunk = lane_is_b ? n0 / 128 : m0 / 128;
+  if (BM == 256) chunk += lane >> 5;
+  const int chunk_max = (lane_is_b ? chunks_b : chunks_a) - 1;
+  chunk = chunk < chunk_max ? chunk : chunk_max;
+  const uint8_t* sc_src = (lane_is_b ? sfb : sfa) + (int64_t)chunk * k_steps * 512 + (lane & 31) * 16;
+  const int sc_dst = (BM == 256 && (wave & 1)) ? kOffSB : kOffSA;
+  static_assert(BM == BN, "the scale staging assumes square tiles");
+  // load number n of a step: n < kLoadsA -> A group, < kLoadsA+kLoadsB -> B group, else scales
+  constexpr int kLoadsPerStep = kLoadsA + kLoadsB + 1;
+  auto fetch_one = [&](int n, int ks, uint8_t* buf) {
+    if (n < kLoadsA) {
+      __builtin_amdgcn_global_load_lds((gptr_t)(A + (int64_t)ks * kBK + offA[n]),
+                                       (lptr_t)(buf + (wave * kLoadsA + n) * kGroupStride), 16, 0, 0);
+    } else if (n < kLoadsA + kLoadsB) {
+      const int i = n - kLoadsA;
+      __builtin_amdgcn_global_load_lds((gptr_t)(B + (int64_t)ks * kBK + offB[i]),
+                                       (lptr_t)(buf + kOffB + (wave * kLoadsB + i) * kGroupStride), 16, 0, 0);
+    } else {
+      __builtin_amdgcn_global_load_lds((gptr_t)(sc_src + (int64_t)ks * 512), (lptr_t)(buf + sc_dst), 16, 0, 0);
     }
+  };
+  auto fetch = [&](int ks, uint8_t* buf) {
+#pragma unroll
+    for (int n = 0; n < kLoadsPerStep; ++n) fetch_one(n, ks, buf);
   };
 
   v4f acc[TM][TN];
@@ -148,47 +155,63 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // (r%32)*16 + (r/32)*4, so the 16 bytes at (r%32)*16 hold the words of rows r%32 + {0,32,64,96},
   // i.e. of the four 16-row tiles t with the same parity.  Two reads per chunk cover its 8 tiles.
   // A word holds the 4 K-block bytes of a row; the lane's own (K-block lane/16) goes to byte 0.
-  auto load_scales = [&](uint32_t scale_off, int row0, int (&sc)[8]) {  // row0: multiple of 128
+  struct ScaleWords {
+    u32x4 even, odd;  // tiles 0,2,4,6 and 1,3,5,7 of a 128-row chunk
+  };
+  auto load_scales = [&](uint32_t scale_off, int row0) -> ScaleWords {  // row0: multiple of 128
     const uint32_t o = scale_off + (row0 >> 7) * 512 + l16 * 16;
-    const u32x4 even = *reinterpret_cast<const u32x4*>(lds + o);        // tiles 0,2,4,6
-    const u32x4 odd = *reinterpret_cast<const u32x4*>(lds + o + 256);   // tiles 1,3,5,7
-    const int sh = kq * 8;
-    sc[0] = even.x >> sh; sc[2] = even.y >> sh; sc[4] = even.z >> sh; sc[6] = even.w >> sh;
-    sc[1] = odd.x >> sh;  sc[3] = odd.y >> sh;  sc[5] = odd.z >> sh;  sc[7] = odd.w >> sh;
+    return ScaleWords{*reinterpret_cast<const u32x4*>(lds + o), *reinterpret_cast<const u32x4*>(lds + o + 256)};
+  };
+  // scale operand of wave tile t (compile-time) out of NT tiles; with 4 tiles per wave the wave
+  // sits in the lower or upper half of its chunk
+  const int scale_shift = kq * 8;
+  auto scale_of = [&](const ScaleWords& w, int t, int nt, bool upper) -> int {
+    auto word = [&](int tile) -> uint32_t {
+      const u32x4& v = (tile & 1) ? w.odd : w.even;
+      const int e = tile >> 1;
+      return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w;
+    };
+    const uint32_t x = nt == 8 ? word(t) : (upper ? word(4 + t) : word(t));
+    return (int)(x >> scale_shift);
   };
   static_assert((TM == 8 || TM == 4) && (TN == 8 || TN == 4), "wave tile is 128 or 64 rows/columns");
 
-  // prologue: step 0 into LDS buffer 0
-  fetch(0, lds);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // prologue: steps 0 .. NST-2 into the first ring slots (clamped for very short K)
+  constexpr int kAhead = NST - 1;  // steps in flight ahead of the one being multiplied
+#pragma unroll
+  for (int p = 0; p < kAhead; ++p) fetch(p < k_steps ? p : k_steps - 1, lds + p * kStageBytes);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kAhead - 1) * kLoadsPerStep) : "memory");
   __syncthreads();
 
+  int slot = 0;  // ring slot of step ks
   for (int ks = 0; ks < k_steps; ++ks) {
-    // Start the loads of the following step (clamped at the end, where the extra load lands in
-    // the idle buffer and is ignored), multiply this step, then wait for the loads and for the
-    // other waves.  The scheduling fences keep the compiler from sinking the MFMAs below the
-    // wait and barrier, which would serialise memory and math.
-    const uint32_t cur = (ks & 1) * kStageBytes;
-    fetch(ks + 1 < k_steps ? ks + 1 : ks, lds + ((ks & 1) ^ 1) * kStageBytes);
+    // Multiply this step while the loads of step ks+NST-1 are issued (clamped at the end, where
+    // the extra loads land in an idle slot and are ignored), then wait for step ks+1 to have
+    // landed and for the other waves.  The scheduling fences pin the order: without them the
+    // compiler sinks the MFMAs below the wait and barrier, which serialises memory and math.
+    const uint32_t cur = slot * kStageBytes;
+    const int slot_load = slot == 0 ? NST - 1 : slot - 1;  // the slot read in the previous step
+    uint8_t* nxt = lds + slot_load * kStageBytes;
+    const int kn = ks + kAhead < k_steps ? ks + kAhead : k_steps - 1;
+    slot = slot + 1 == NST ? 0 : slot + 1;
     __builtin_amdgcn_sched_barrier(0);
 
-    int sa[8], sb[8];
     v8i fb[TN];
-    load_scales(cur + kOffSB, (wn * WN) & ~127, sb);
-    load_scales(cur + kOffSA, (wm * WM) & ~127, sa);
-    if constexpr (TM == 4) {  // 64-row wave tile: the upper half of a chunk starts at tile 4
-      const bool upper = (wm & 1) != 0;
+    const ScaleWords swb = load_scales(cur + kOffSB, (wn * WN) & ~127);
+    const ScaleWords swa = load_scales(cur + kOffSA, (wm * WM) & ~127);
+    int sa[TM], sb[TN];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) sa[i] = upper ? sa[4 + i] : sa[i];
-    }
-    if constexpr (TN == 4) {
-      const bool upper = (wn & 1) != 0;
+    for (int t = 0; t < TM; ++t) sa[t] = scale_of(swa, t, TM, (wm & 1) != 0);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) sb[j] = upper ? sb[4 + j] : sb[j];
-    }
+    for (int t = 0; t < TN; ++t) sb[t] = scale_of(swb, t, TN, (wn & 1) != 0);
 #pragma unroll
     for (int t = 0; t < TN; ++t) fb[t] = load_frag(cur + kOffB, wn * WN + t * 16);
     v8i fa = load_frag(cur, wm * WM);
+    __builtin_amdgcn_sched_barrier(0);
+    // With one wave per SIMD nothing else hides instruction issue, so the loads of the next
+    // step are slipped in one at a time behind MFMAs (each MFMA keeps the pipe busy for 8
+    // passes while the wave issues something else).
+    int n_load = 0;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       v8i fa_next = fa;
@@ -197,12 +220,20 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
       for (int j = 0; j < TN; ++j) {
         // B fragment as the row operand: acc[i][j][v] = D[m = l16][n = 4*kq + v] of the tile
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], fa, acc[i][j], 0, 0, 0, sb[j], 0, sa[i]);
+        if (n_load < kLoadsPerStep && (i * TN + j) % 2 == 0) {
+          fetch_one(n_load, kn, nxt);
+          ++n_load;
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
       fa = fa_next;
       __builtin_amdgcn_sched_barrier(0);
     }
-    // the next step's panels must have landed, and every wave must be done reading `cur`
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (; n_load < kLoadsPerStep; ++n_load) fetch_one(n_load, kn, nxt);
+    // the next step's panels must have landed (later ones may still be in flight), and every
+    // wave must be done reading `cur`
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kAhead - 1) * kLoadsPerStep) : "memory");
     __syncthreads();
   }
 
@@ -223,12 +254,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST>
 int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N,
                 int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream) {
   const int tiles_m = (int)ceil_div(M, BM), tiles_n = (int)ceil_div(N, BN);
-  const size_t lds_bytes = (size_t)2 * (((BM + BN) / kGroupRows) * kGroupStride + ((BM + BN) / 128) * 512);  // two K-steps
-  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N>;
+  size_t lds_bytes = (size_t)NST * (((BM + BN) / kGroupRows) * kGroupStride + ((BM + BN) / 128) * 512);  // NST K-steps
+  // A grid that fits the chip once should land one workgroup per CU: asking for more than half
+  // of the LDS keeps the dispatcher from pairing two workgroups on one CU while others idle.
+  if ((int64_t)tiles_m * tiles_n <= device_facts().cu_count && lds_bytes < 82 * 1024) lds_bytes = 82 * 1024;
+  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST>;
   if (lds_bytes > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess)
@@ -258,6 +292,6 @@ extern "C" int dt_mx_fp8_bf16(const void* a, const void* b, const uint8_t* sfa, 
   const int variant = dt::tuning("gemm.variant");
   const int64_t tiles256 = dt::ceil_div(M, 256) * dt::ceil_div(N, 256);
   const bool big = variant == 2 || (variant == 0 && tiles256 >= dt::device_facts().cu_count / 2);
-  if (big) return dt::launch_gemm<256, 256, 2, 2>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
-  return dt::launch_gemm<128, 128, 2, 2>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  if (big) return dt::launch_gemm<256, 256, 2, 2, 2>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  return dt::launch_gemm<128, 128, 2, 2, 4>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
 }
