@@ -246,7 +246,8 @@ def extra_kernels(torch, cabi, util, dev, K, W):
     b_data, sfb = cabi.mx_fp8_quantize(b, 1, False, e4, cabi.SCALE_BLOCKED)
     out = torch.empty((M, N), dtype=bf16, device=dev)
     del a, b
-    us = time_launches(lambda i: cabi.mx_fp8_bf16(a_data, b_data, sfa, sfb, out), 1, max(5, K // 5), max(2, W // 5))
+    # the clocks take tens of milliseconds of sustained MFMA load to settle: warm up for ~30 launches
+    us = time_launches(lambda i: cabi.mx_fp8_bf16(a_data, b_data, sfa, sfb, out), 1, max(20, K // 2), max(30, W))
     flops = 2.0 * M * N * Kd
     tf = flops / (us * 1e-6) / 1e12
     rows.append({"kernel": "mx_fp8_bf16", "workload": "config 5: 8192^3 e4m3 x e4m3, E8M0 block-32 scales -> bf16",

@@ -46,7 +46,7 @@ __device__ __forceinline__ int64_t sf_group_offset(int r, int ks, int k_steps) {
   return ((int64_t)(r >> 7) * k_steps + ks) * 512 + (r & 31) * 16 + ((r & 127) >> 5) * 4;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int FIRST, int EVERY>
 __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const uint8_t* __restrict__ sfa,
     const uint8_t* __restrict__ sfb, int M, int N, int K, int64_t lda, int64_t ldb, uint16_t* __restrict__ out,
@@ -118,6 +118,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   static_assert(BM == BN, "the scale staging assumes square tiles");
   // load number n of a step: n < kLoadsA -> A group, < kLoadsA+kLoadsB -> B group, else scales
   constexpr int kLoadsPerStep = kLoadsA + kLoadsB + 1;
+  constexpr int kFirstLoadAfter = FIRST;  // MFMAs issued before the first slipped-in load
+  static_assert(TM == TN, "the MFMA schedule assumes a square wave tile");
   auto fetch_one = [&](int n, int ks, uint8_t* buf) {
     if (n < kLoadsA) {
       __builtin_amdgcn_global_load_lds((gptr_t)(A + (int64_t)ks * kBK + offA[n]),
@@ -199,35 +201,48 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     v8i fb[TN];
     const ScaleWords swb = load_scales(cur + kOffSB, (wn * WN) & ~127);
     const ScaleWords swa = load_scales(cur + kOffSA, (wm * WM) & ~127);
+    // Expanding-square order: step k of the schedule loads fragments a[k+1], b[k+1] and issues
+    // the 2k+1 MFMAs that a[k], b[k] make possible, so the first MFMA waits for two fragments
+    // only and the LDS burst after the barrier overlaps with math.  With one wave per SIMD
+    // nothing else hides instruction issue, so the global->LDS loads of the step ahead are
+    // slipped in one at a time behind MFMAs (an MFMA keeps the pipe busy for 8 passes while
+    // the wave issues something else).  sched_barrier pins this order.
+    v8i fa[TM];
+    fa[0] = load_frag(cur, wm * WM);
+    fb[0] = load_frag(cur + kOffB, wn * WN);
+    if (TM > 1) {
+      fa[1] = load_frag(cur, wm * WM + 16);
+      fb[1] = load_frag(cur + kOffB, wn * WN + 16);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     int sa[TM], sb[TN];
 #pragma unroll
     for (int t = 0; t < TM; ++t) sa[t] = scale_of(swa, t, TM, (wm & 1) != 0);
 #pragma unroll
     for (int t = 0; t < TN; ++t) sb[t] = scale_of(swb, t, TN, (wn & 1) != 0);
-#pragma unroll
-    for (int t = 0; t < TN; ++t) fb[t] = load_frag(cur + kOffB, wn * WN + t * 16);
-    v8i fa = load_frag(cur, wm * WM);
     __builtin_amdgcn_sched_barrier(0);
-    // With one wave per SIMD nothing else hides instruction issue, so the loads of the next
-    // step are slipped in one at a time behind MFMAs (each MFMA keeps the pipe busy for 8
-    // passes while the wave issues something else).
-    int n_load = 0;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      v8i fa_next = fa;
-      if (i + 1 < TM) fa_next = load_frag(cur, wm * WM + (i + 1) * 16);
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        // B fragment as the row operand: acc[i][j][v] = D[m = l16][n = 4*kq + v] of the tile
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], fa, acc[i][j], 0, 0, 0, sb[j], 0, sa[i]);
-        if (n_load < kLoadsPerStep && (i * TN + j) % 2 == 0) {
-          fetch_one(n_load, kn, nxt);
-          ++n_load;
-          __builtin_amdgcn_sched_barrier(0);
-        }
+    int n_load = 0, n_mfma = 0;
+    auto mfma = [&](int i, int j) {
+      // B fragment as the row operand: acc[i][j][v] = D[m = l16][n = 4*kq + v] of the tile
+      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], fa[i], acc[i][j], 0, 0, 0, sb[j], 0, sa[i]);
+      if (n_load < kLoadsPerStep && n_mfma >= kFirstLoadAfter && (n_mfma - kFirstLoadAfter) % EVERY == 0) {
+        fetch_one(n_load, kn, nxt);
+        ++n_load;
       }
-      fa = fa_next;
+      ++n_mfma;
       __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int k = 0; k < TM; ++k) {
+      if (k + 2 < TM) {
+        fa[k + 2] = load_frag(cur, wm * WM + (k + 2) * 16);
+        fb[k + 2] = load_frag(cur + kOffB, wn * WN + (k + 2) * 16);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int j = 0; j <= k; ++j) mfma(k, j);
+#pragma unroll
+      for (int i = 0; i < k; ++i) mfma(i, k);
     }
 #pragma unroll
     for (; n_load < kLoadsPerStep; ++n_load) fetch_one(n_load, kn, nxt);
@@ -254,7 +269,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int FIRST, int EVERY>
 int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N,
                 int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream) {
   const int tiles_m = (int)ceil_div(M, BM), tiles_n = (int)ceil_div(N, BN);
@@ -262,7 +277,7 @@ int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const ui
   // A grid that fits the chip once should land one workgroup per CU: asking for more than half
   // of the LDS keeps the dispatcher from pairing two workgroups on one CU while others idle.
   if ((int64_t)tiles_m * tiles_n <= device_facts().cu_count && lds_bytes < 82 * 1024) lds_bytes = 82 * 1024;
-  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST>;
+  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST, FIRST, EVERY>;
   if (lds_bytes > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess)
@@ -292,6 +307,7 @@ extern "C" int dt_mx_fp8_bf16(const void* a, const void* b, const uint8_t* sfa, 
   const int variant = dt::tuning("gemm.variant");
   const int64_t tiles256 = dt::ceil_div(M, 256) * dt::ceil_div(N, 256);
   const bool big = variant == 2 || (variant == 0 && tiles256 >= dt::device_facts().cu_count / 2);
-  if (big) return dt::launch_gemm<256, 256, 2, 2, 2>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
-  return dt::launch_gemm<128, 128, 2, 2, 4>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  // <tile M, tile N, waves M, waves N, LDS ring slots, first slipped-in load after MFMA #, one every # MFMAs>
+  if (big) return dt::launch_gemm<256, 256, 2, 2, 2, 0, 2>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  return dt::launch_gemm<128, 128, 2, 2, 4, 1, 2>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
 }
