@@ -28,28 +28,20 @@ int launch_mx(const MxArgs& a) {
                                                                  a.data, a.scale);
     return launch_status();
   }
-  if (a.axis == 0 && x_vec && a.cols % kV == 0 && aligned(a.data, 16) && aligned(a.scale, 8) &&
-      a.rows < (1ll << 31) && a.cols < (1ll << 31) && (LAYOUT == DT_SCALE_PLAIN || a.transpose)) {
+  if (a.axis == 0 && a.transpose && x_vec && a.cols % 4 == 0 && (a.cols * InTraits<IN>::kBytes) % 16 == 0 &&
+      aligned(a.data, 16) && aligned(a.scale, 4) && a.rows < (1ll << 31) && a.cols < (1ll << 31)) {
+    const int64_t tiles = ceil_div(a.rows, (int64_t)kColTRows) * ceil_div(a.cols, (int64_t)kColTCols);
+    if (tiles <= 0x7FFFFFFFll) {
+      mx_col_t_kernel<IN, OUT, LAYOUT><<<(unsigned)tiles, kBlock, 0, a.stream>>>(a.x, (uint32_t)a.rows, (uint32_t)a.cols,
+                                                                              a.data, a.scale);
+      return launch_status();
+    }
+  }
+  if (a.axis == 0 && !a.transpose && x_vec && a.cols % kV == 0 && aligned(a.data, 16) && aligned(a.scale, 8) &&
+      a.rows < (1ll << 31) && a.cols < (1ll << 31) && LAYOUT == DT_SCALE_PLAIN) {
     const int64_t row_tiles = a.rows / 32, col_tiles = ceil_div(a.cols, (int64_t)kWave * kV);
-    auto waves_for = [&](int rbw) { return ceil_div(row_tiles, rbw) * col_tiles; };
-    int rbw = 1;
-    if (a.transpose) {
-      const int64_t enough = (int64_t)cus * 8;
-      int knob = tuning("mx.col_rbw");
-      rbw = knob ? knob : (waves_for(4) >= enough ? 4 : waves_for(2) >= enough ? 2 : 1);
-    }
-    const unsigned grid = (unsigned)ceil_div(waves_for(rbw), kBlock / kWave);
-    const uint32_t R = (uint32_t)a.rows, C = (uint32_t)a.cols;
-    if (!a.transpose) {
-      if constexpr (LAYOUT == DT_SCALE_PLAIN)
-        mx_col_kernel<IN, OUT, false, DT_SCALE_PLAIN, 1><<<grid, kBlock, 0, a.stream>>>(a.x, R, C, a.data, a.scale);
-    } else if (rbw == 4) {
-      mx_col_kernel<IN, OUT, true, LAYOUT, 4><<<grid, kBlock, 0, a.stream>>>(a.x, R, C, a.data, a.scale);
-    } else if (rbw == 2) {
-      mx_col_kernel<IN, OUT, true, LAYOUT, 2><<<grid, kBlock, 0, a.stream>>>(a.x, R, C, a.data, a.scale);
-    } else {
-      mx_col_kernel<IN, OUT, true, LAYOUT, 1><<<grid, kBlock, 0, a.stream>>>(a.x, R, C, a.data, a.scale);
-    }
+    const unsigned grid = (unsigned)ceil_div(row_tiles * col_tiles, kBlock / kWave);
+    mx_col_kernel<IN, OUT><<<grid, kBlock, 0, a.stream>>>(a.x, (uint32_t)a.rows, (uint32_t)a.cols, a.data, a.scale);
     return launch_status();
   }
   // general orientation / alignment

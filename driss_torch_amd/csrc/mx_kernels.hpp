@@ -3,12 +3,16 @@
 //  mx_row_kernel   blocks along rows.  A 32-element block is spread over 4 lanes (16-bit
 //                  input, 8 elements per 16-byte load) or 8 lanes (fp32 input); the block
 //                  maximum is an integer max over DPP quad/row permutes -- no LDS.
-//  mx_col_kernel   blocks down columns.  A lane owns 8 (fp32: 4) adjacent columns of a
-//                  32-row tile, so the block maximum needs no cross-lane traffic at all;
-//                  the payload is written in the input orientation or transposed.
+//  mx_col_kernel   blocks down columns, payload in the input orientation.  A lane owns 8
+//                  (fp32: 4) adjacent columns of a 32-row tile, so the block maximum needs
+//                  no cross-lane traffic at all.
+//  mx_col_t_kernel blocks down columns, payload transposed through LDS so that the stores
+//                  are full 128-byte rows of the [cols, rows] output.
 //  mx_any_kernel   one thread per block, arbitrary strides: covers every (axis, transpose)
 //                  pair and shapes the fast kernels do not take.
 #pragma once
+
+#include <type_traits>
 
 #include "dt_device.hpp"
 #include "dt_host.hpp"
@@ -160,134 +164,192 @@ __global__ __launch_bounds__(kBlock) void mx_row_kernel(const void* __restrict__
 }
 
 // --------------------------------------------------------------- blocks down columns
-// One wave owns RBW consecutive 32-row tiles of 64*kV columns.  TRANSPOSE writes the payload
-// as [cols, rows] (32 contiguous bytes per column and tile) and the scales as
-// [cols, rows/32]; otherwise payload [rows, cols] and scales [rows/32, cols].
-template <int IN, int OUT, bool TRANSPOSE, int LAYOUT, int RBW>
+// In-place payload: one wave owns a 32-row tile of 64*kV columns; a lane holds kV adjacent
+// columns x 32 rows in registers.  Payload [rows, cols], scales [rows/32, cols].
+template <int IN, int OUT>
 __global__ __launch_bounds__(kBlock) void mx_col_kernel(const void* __restrict__ x, uint32_t rows, uint32_t cols,
                                                         uint8_t* __restrict__ data, uint8_t* __restrict__ scale) {
   constexpr int kV = InTraits<IN>::kVec;   // columns per lane
   constexpr int kW = kV / 4;               // fp8 words per lane and row: 2 or 1
   const int lane = threadIdx.x % kWave;
-  const uint32_t row_tiles = rows / 32u, rb_groups = (row_tiles + RBW - 1) / RBW;
+  const uint32_t row_tiles = rows / 32u;
   const uint32_t col_tiles = (cols + kWave * kV - 1) / (kWave * kV);
   const uint32_t wave_id = (blockIdx.x * kBlock + threadIdx.x) / kWave;
-  if (wave_id >= rb_groups * col_tiles) return;  // whole wave leaves; no barrier in this kernel
+  if (wave_id >= row_tiles * col_tiles) return;  // whole wave leaves; no barrier in this kernel
   // consecutive waves walk down the rows first so a workgroup covers adjacent row tiles
-  const uint32_t ct = wave_id / rb_groups, rg = wave_id - ct * rb_groups;
+  const uint32_t ct = wave_id / row_tiles, rb = wave_id - ct * row_tiles;
   const uint32_t col0 = ct * (kWave * kV) + lane * kV;
   if (col0 >= cols) return;  // cols % kV == 0, so a lane is either fully inside or outside
   const uint32_t row_vecs = cols / kV;
   const u32x4* v = static_cast<const u32x4*>(x);
-  uint32_t sbytes[kV];  // per column: RBW scale bytes packed (TRANSPOSE only)
+  const uint64_t vfirst = (uint64_t)rb * 32u * row_vecs + col0 / kV;
+  u32x4 w[32];
 #pragma unroll
-  for (int c = 0; c < kV; ++c) sbytes[c] = 0;
+  for (int i = 0; i < 32; ++i) w[i] = ld_stream(v + vfirst + (uint64_t)i * row_vecs);
 
+  // per-column magnitude maxima
+  uint32_t cm[kV];
+  if constexpr (IN == DT_BF16) {
+    uint32_t p0 = 0, p1 = 0, p2 = 0, p3 = 0;
 #pragma unroll
-  for (int t = 0; t < RBW; ++t) {
-    const uint32_t rb = rg * RBW + t;
-    if (rb >= row_tiles) break;
-    const uint64_t vfirst = (uint64_t)rb * 32u * row_vecs + col0 / kV;
-    u32x4 w[32];
+    for (int i = 0; i < 32; ++i) {
+      p0 = pk_absmax16(p0, w[i].x); p1 = pk_absmax16(p1, w[i].y);
+      p2 = pk_absmax16(p2, w[i].z); p3 = pk_absmax16(p3, w[i].w);
+    }
+    cm[0] = p0 << 16; cm[1] = p0 & 0xFFFF0000u; cm[2] = p1 << 16; cm[3] = p1 & 0xFFFF0000u;
+    cm[4] = p2 << 16; cm[5] = p2 & 0xFFFF0000u; cm[6] = p3 << 16; cm[7] = p3 & 0xFFFF0000u;
+  } else if constexpr (IN == DT_F16) {
 #pragma unroll
-    for (int i = 0; i < 32; ++i) w[i] = ld_stream(v + vfirst + (uint64_t)i * row_vecs);
-
-    // per-column magnitude maxima
-    uint32_t cm[kV];
-    if constexpr (IN == DT_BF16) {
-      uint32_t p0 = 0, p1 = 0, p2 = 0, p3 = 0;
+    for (int c = 0; c < 8; ++c) cm[c] = 0;
 #pragma unroll
-      for (int i = 0; i < 32; ++i) {
-        p0 = pk_absmax16(p0, w[i].x); p1 = pk_absmax16(p1, w[i].y);
-        p2 = pk_absmax16(p2, w[i].z); p3 = pk_absmax16(p3, w[i].w);
-      }
-      cm[0] = p0 << 16; cm[1] = p0 & 0xFFFF0000u; cm[2] = p1 << 16; cm[3] = p1 & 0xFFFF0000u;
-      cm[4] = p2 << 16; cm[5] = p2 & 0xFFFF0000u; cm[6] = p3 << 16; cm[7] = p3 & 0xFFFF0000u;
-    } else if constexpr (IN == DT_F16) {
+    for (int i = 0; i < 32; ++i) {
+      float f[8];
+      unpack8<IN>(w[i], f);
 #pragma unroll
-      for (int c = 0; c < 8; ++c) cm[c] = 0;
+      for (int c = 0; c < 8; ++c) cm[c] = umax(cm[c], absbits_f32(as_u32(f[c])));
+    }
+  } else {
+    cm[0] = cm[1] = cm[2] = cm[3] = 0;
 #pragma unroll
-      for (int i = 0; i < 32; ++i) {
-        float f[8];
-        unpack8<IN>(w[i], f);
+    for (int i = 0; i < 32; ++i) {
+      cm[0] = umax(cm[0], absbits_f32(w[i].x)); cm[1] = umax(cm[1], absbits_f32(w[i].y));
+      cm[2] = umax(cm[2], absbits_f32(w[i].z)); cm[3] = umax(cm[3], absbits_f32(w[i].w));
+    }
+  }
+  float mult[kV];
+  bool nanc[kV];
+  uint32_t byte_lo = 0, byte_hi = 0;  // the kV scale bytes packed in column order
 #pragma unroll
-        for (int c = 0; c < 8; ++c) cm[c] = umax(cm[c], absbits_f32(as_u32(f[c])));
-      }
+  for (int c = 0; c < kV; ++c) {
+    const MxScale<OUT> s = mx_scale_from_absbits<OUT>(cm[c]);
+    mult[c] = s.mult;
+    nanc[c] = s.nan;
+    if (c < 4) byte_lo |= s.byte << (8 * c); else byte_hi |= s.byte << (8 * (c - 4));
+  }
+  auto elem = [&](int i, int c) -> float {
+    if constexpr (IN == DT_F32) {
+      return as_f32(c == 0 ? w[i].x : c == 1 ? w[i].y : c == 2 ? w[i].z : w[i].w);
     } else {
-      cm[0] = cm[1] = cm[2] = cm[3] = 0;
-#pragma unroll
-      for (int i = 0; i < 32; ++i) {
-        cm[0] = umax(cm[0], absbits_f32(w[i].x)); cm[1] = umax(cm[1], absbits_f32(w[i].y));
-        cm[2] = umax(cm[2], absbits_f32(w[i].z)); cm[3] = umax(cm[3], absbits_f32(w[i].w));
-      }
+      const uint32_t d = (c >> 1) == 0 ? w[i].x : (c >> 1) == 1 ? w[i].y : (c >> 1) == 2 ? w[i].z : w[i].w;
+      if constexpr (IN == DT_BF16) return (c & 1) ? bf16_hi(d) : bf16_lo(d);
+      else return (c & 1) ? f16_hi(d) : f16_lo(d);
     }
-    float mult[kV];
-    bool nanc[kV];
-    uint32_t byte_lo = 0, byte_hi = 0;  // the kV scale bytes packed in column order
+  };
+  uint8_t* drow = data + (uint64_t)rb * 32u * cols + col0;
 #pragma unroll
-    for (int c = 0; c < kV; ++c) {
-      const MxScale<OUT> s = mx_scale_from_absbits<OUT>(cm[c]);
-      mult[c] = s.mult;
-      nanc[c] = s.nan;
-      if (c < 4) byte_lo |= s.byte << (8 * c); else byte_hi |= s.byte << (8 * (c - 4));
-      sbytes[c] |= s.byte << (8 * t);
+  for (int i = 0; i < 32; ++i) {
+    uint32_t r[kW];
+#pragma unroll
+    for (int q = 0; q < kW; ++q) {
+      r[q] = pack4_finite<OUT>(elem(i, 4 * q) * mult[4 * q], elem(i, 4 * q + 1) * mult[4 * q + 1],
+                               elem(i, 4 * q + 2) * mult[4 * q + 2], elem(i, 4 * q + 3) * mult[4 * q + 3]);
+      uint32_t nanmask = (nanc[4 * q] ? 0xFFu : 0u) | (nanc[4 * q + 1] ? 0xFF00u : 0u) |
+                         (nanc[4 * q + 2] ? 0xFF0000u : 0u) | (nanc[4 * q + 3] ? 0xFF000000u : 0u);
+      r[q] = (r[q] & ~nanmask) | (0x7F7F7F7Fu & nanmask);
     }
+    if constexpr (kW == 2) st_stream(reinterpret_cast<u32x2*>(drow + (uint64_t)i * cols), u32x2{r[0], r[1]});
+    else st_stream(reinterpret_cast<uint32_t*>(drow + (uint64_t)i * cols), r[0]);
+  }
+  // scales [rows/32, cols]: kV adjacent bytes
+  uint8_t* srow = scale + (uint64_t)rb * cols + col0;
+  if constexpr (kW == 2) *reinterpret_cast<u32x2*>(srow) = u32x2{byte_lo, byte_hi};
+  else *reinterpret_cast<uint32_t*>(srow) = byte_lo;
+}
+
+// ------------------------------------------- blocks down columns, transposed payload
+// A workgroup owns 128 rows x 256 columns.  Wave w takes the 32-row tile w: a lane holds 4
+// adjacent columns x 32 rows in registers (8- or 16-byte loads), so the block maximum is again
+// lane-local, and converts column by column (4 consecutive rows per packed word).  The fp8
+// bytes go to LDS as [column][128 rows] and leave as full 128-byte rows of the [cols, rows]
+// output; the 4 scale bytes of a column (one per wave) leave as one word.
+constexpr int kColTRows = 128, kColTCols = 256, kColTPitch = 144;  // LDS row pitch: 128 + 16 pad
+template <int IN, int OUT, int LAYOUT>
+__global__ __launch_bounds__(kBlock) void mx_col_t_kernel(const void* __restrict__ x, uint32_t rows, uint32_t cols,
+                                                          uint8_t* __restrict__ data, uint8_t* __restrict__ scale) {
+  constexpr int kB = InTraits<IN>::kBytes;
+  __shared__ __attribute__((aligned(16))) uint8_t tile[kColTCols * kColTPitch];
+  __shared__ __attribute__((aligned(16))) uint32_t stile[kColTCols];  // 4 scale bytes per column
+  const int tid = threadIdx.x, lane = tid % kWave, w = tid / kWave;
+  // consecutive workgroups walk down the rows, so their 128-byte output segments are adjacent
+  // (measured 7% faster than walking along the columns)
+  const uint32_t row_tiles128 = (rows + kColTRows - 1) / kColTRows;
+  const uint32_t tc = blockIdx.x / row_tiles128, tr = blockIdx.x - tc * row_tiles128;
+  const uint32_t row0 = tr * kColTRows + w * 32, col0 = tc * kColTCols + lane * 4;
+  const bool active = row0 < rows && col0 < cols;  // rows % 32 == 0 and cols % 4 == 0
+
+  uint32_t sbyte[4] = {0, 0, 0, 0};
+  if (active) {
+    // 32 rows x 4 columns kept packed as loaded: fp32 -> one 16-byte load per row, 16-bit -> one
+    // 8-byte load; elements are unpacked where they are used
+    typedef typename std::conditional<IN == DT_F32, u32x4, u32x2>::type row_t;
+    row_t wv[32];
+    uint32_t cm[4] = {0, 0, 0, 0};
+    const uint8_t* p = static_cast<const uint8_t*>(x) + ((uint64_t)row0 * cols + col0) * kB;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) wv[i] = ld_stream(reinterpret_cast<const row_t*>(p + (uint64_t)i * cols * kB));
     auto elem = [&](int i, int c) -> float {
       if constexpr (IN == DT_F32) {
-        return as_f32(c == 0 ? w[i].x : c == 1 ? w[i].y : c == 2 ? w[i].z : w[i].w);
+        return as_f32(c == 0 ? wv[i].x : c == 1 ? wv[i].y : c == 2 ? wv[i].z : wv[i].w);
       } else {
-        const uint32_t d = (c >> 1) == 0 ? w[i].x : (c >> 1) == 1 ? w[i].y : (c >> 1) == 2 ? w[i].z : w[i].w;
+        const uint32_t d = c < 2 ? wv[i].x : wv[i].y;
         if constexpr (IN == DT_BF16) return (c & 1) ? bf16_hi(d) : bf16_lo(d);
         else return (c & 1) ? f16_hi(d) : f16_lo(d);
       }
     };
-    if constexpr (!TRANSPOSE) {
-      uint8_t* drow = data + (uint64_t)rb * 32u * cols + col0;
+    if constexpr (IN == DT_BF16) {
+      uint32_t p0 = 0, p1 = 0;
 #pragma unroll
-      for (int i = 0; i < 32; ++i) {
-        uint32_t r[kW];
-#pragma unroll
-        for (int q = 0; q < kW; ++q) {
-          r[q] = pack4_finite<OUT>(elem(i, 4 * q) * mult[4 * q], elem(i, 4 * q + 1) * mult[4 * q + 1],
-                                   elem(i, 4 * q + 2) * mult[4 * q + 2], elem(i, 4 * q + 3) * mult[4 * q + 3]);
-          uint32_t nanmask = (nanc[4 * q] ? 0xFFu : 0u) | (nanc[4 * q + 1] ? 0xFF00u : 0u) |
-                             (nanc[4 * q + 2] ? 0xFF0000u : 0u) | (nanc[4 * q + 3] ? 0xFF000000u : 0u);
-          r[q] = (r[q] & ~nanmask) | (0x7F7F7F7Fu & nanmask);
-        }
-        if constexpr (kW == 2) st_stream(reinterpret_cast<u32x2*>(drow + (uint64_t)i * cols), u32x2{r[0], r[1]});
-        else st_stream(reinterpret_cast<uint32_t*>(drow + (uint64_t)i * cols), r[0]);
-      }
-      // scales [rows/32, cols]: kV adjacent bytes
-      uint8_t* srow = scale + (uint64_t)rb * cols + col0;
-      if constexpr (kW == 2) *reinterpret_cast<u32x2*>(srow) = u32x2{byte_lo, byte_hi};
-      else *reinterpret_cast<uint32_t*>(srow) = byte_lo;
+      for (int i = 0; i < 32; ++i) { p0 = pk_absmax16(p0, wv[i].x); p1 = pk_absmax16(p1, wv[i].y); }
+      cm[0] = p0 << 16; cm[1] = p0 & 0xFFFF0000u; cm[2] = p1 << 16; cm[3] = p1 & 0xFFFF0000u;
     } else {
 #pragma unroll
-      for (int c = 0; c < kV; ++c) {
-        uint32_t r[8];
+      for (int i = 0; i < 32; ++i)
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-          r[q] = pack4_finite<OUT>(elem(4 * q, c) * mult[c], elem(4 * q + 1, c) * mult[c],
-                                   elem(4 * q + 2, c) * mult[c], elem(4 * q + 3, c) * mult[c]);
-          if (nanc[c]) r[q] = 0x7F7F7F7Fu;
-        }
-        u32x4* dcol = reinterpret_cast<u32x4*>(data + (uint64_t)(col0 + c) * rows + (uint64_t)rb * 32u);
-        // plain stores: neighbouring tiles complete these 128-byte lines in the L2
-        dcol[0] = u32x4{r[0], r[1], r[2], r[3]};
-        dcol[1] = u32x4{r[4], r[5], r[6], r[7]};
+        for (int c = 0; c < 4; ++c) cm[c] = umax(cm[c], absbits_f32(as_u32(elem(i, c))));
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const MxScale<OUT> s = mx_scale_from_absbits<OUT>(cm[c]);
+      sbyte[c] = s.byte;
+      uint32_t r[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        r[q] = pack4_finite<OUT>(elem(4 * q, c) * s.mult, elem(4 * q + 1, c) * s.mult, elem(4 * q + 2, c) * s.mult,
+                                 elem(4 * q + 3, c) * s.mult);
+        if (s.nan) r[q] = 0x7F7F7F7Fu;
       }
+      u32x4* t = reinterpret_cast<u32x4*>(tile + (lane * 4 + c) * kColTPitch + w * 32);
+      t[0] = u32x4{r[0], r[1], r[2], r[3]};
+      t[1] = u32x4{r[4], r[5], r[6], r[7]};
     }
   }
-  if constexpr (TRANSPOSE) {
-    // scales [cols, rows/32]: this wave's RBW bytes per column are adjacent
-    const uint32_t rb0 = rg * RBW;
 #pragma unroll
-    for (int c = 0; c < kV; ++c) {
+  for (int c = 0; c < 4; ++c) reinterpret_cast<uint8_t*>(stile)[(lane * 4 + c) * 4 + w] = (uint8_t)sbyte[c];
+  __syncthreads();
+
+  // 256 output rows (columns of x) x 8 chunks of 16 bytes; 8 consecutive lanes write one row
+  const uint32_t trow0 = tr * kColTRows, tcol0 = tc * kColTCols;
 #pragma unroll
-      for (int t = 0; t < RBW; ++t) {
-        if (rb0 + t < row_tiles)
-          scale[scale_offset<LAYOUT>(col0 + c, rb0 + t, row_tiles)] = (uint8_t)(sbytes[c] >> (8 * t));
-      }
+  for (int i = 0; i < kColTCols * 8 / kBlock; ++i) {
+    const int id = tid + i * kBlock, r = id >> 3, q = id & 7;
+    if (tcol0 + r < cols && trow0 + q * 16 < rows) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(tile + r * kColTPitch + q * 16);
+      st_stream(reinterpret_cast<u32x4*>(data + (uint64_t)(tcol0 + r) * rows + trow0 + q * 16), v);
+    }
+  }
+  // scales [cols, rows/32]: 4 bytes per column of this tile
+  const uint32_t RB = rows / 32, rb0 = tr * 4;
+  if (tcol0 + tid < cols) {
+    const uint32_t sw = stile[tid];
+    const uint32_t c = tcol0 + tid;
+    if (LAYOUT == DT_SCALE_BLOCKED || (RB % 4 == 0)) {
+      // rb0 % 4 == 0: the four bytes are adjacent and word aligned in both layouts (bytes of
+      // row tiles past the end are zero, which is what the padding must hold)
+      *reinterpret_cast<uint32_t*>(scale + scale_offset<LAYOUT>(c, rb0, RB)) = sw;
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (rb0 + k < RB) scale[scale_offset<LAYOUT>(c, rb0 + k, RB)] = (uint8_t)(sw >> (8 * k));
     }
   }
 }
