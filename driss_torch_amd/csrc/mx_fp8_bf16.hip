@@ -58,7 +58,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int kGroupsA = BM / kGroupRows, kGroupsB = BN / kGroupRows;
   constexpr int kPanelA = kGroupsA * kGroupStride, kPanelB = kGroupsB * kGroupStride;
-  constexpr int kScaleA = (BM / 128) * 512, kScaleB = (BN / 128) * 512;  // blocked scale chunks of one K-step
+  constexpr int kScaleA = 1024, kScaleB = 1024;  // up to two 512-byte blocked scale chunks of one K-step each
   constexpr int kOffB = kPanelA, kOffSA = kPanelA + kPanelB, kOffSB = kOffSA + kScaleA;
   constexpr int kStageBytes = kOffSB + kScaleB;  // one K-step: A panel, B panel, A scales, B scales
   constexpr int kWaves = WAVES_M * WAVES_N;
@@ -103,36 +103,42 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     gr = gr < N ? gr : N - 1;
     offB[i] = (uint32_t)((int64_t)gr * ldb + lchunk * 16);
   }
-  // Scales: one more wave-wide load per step.  256-row tiles: even waves bring the two A chunks
-  // (lanes 0-31 / 32-63), odd waves the two B chunks; 128-row tiles: lanes 0-31 bring the A
-  // chunk and lanes 32-63 the B chunk.  Every wave issues it (duplicates write identical bytes),
-  // which keeps the instruction stream free of branches.
-  const int chunks_a = (M + 127) / 128, chunks_b = (N + 127) / 128;
-  const bool lane_is_b = (BM == 256) ? (wave & 1) != 0 : lane >= 32;
-  int chunk = lane_is_b ? n0 / 128 : m0 / 128;
-  if (BM == 256) chunk += lane >> 5;
-  const int chunk_max = (lane_is_b ? chunks_b : chunks_a) - 1;
+  // Scales: one more wave-wide load per step.  Even waves bring A chunks, odd waves B chunks:
+  // lanes 0-31 the tile's first 128-row chunk, lanes 32-63 the next one (the second chunk of a
+  // 256-row tile; for a 128-row tile it lands in an unused half of the slot).  Every wave issues
+  // it (duplicates write identical bytes), which keeps the instruction stream free of branches.
+  const bool wave_is_b = (wave & 1) != 0;
+  const int chunk_max = (wave_is_b ? (N + 127) / 128 : (M + 127) / 128) - 1;
+  int chunk = (wave_is_b ? n0 : m0) / 128 + (lane >> 5);
   chunk = chunk < chunk_max ? chunk : chunk_max;
-  const uint8_t* sc_src = (lane_is_b ? sfb : sfa) + (int64_t)chunk * k_steps * 512 + (lane & 31) * 16;
-  const int sc_dst = (BM == 256 && (wave & 1)) ? kOffSB : kOffSA;
-  static_assert(BM == BN, "the scale staging assumes square tiles");
+  const uint8_t* sc_base = wave_is_b ? sfb : sfa;
+  const uint32_t sc_off = (uint32_t)((int64_t)chunk * k_steps * 512 + (lane & 31) * 16);
+  const int sc_dst = wave_is_b ? kOffSB : kOffSA;
   // load number n of a step: n < kLoadsA -> A group, < kLoadsA+kLoadsB -> B group, else scales
   constexpr int kLoadsPerStep = kLoadsA + kLoadsB + 1;
   constexpr int kFirstLoadAfter = FIRST;  // MFMAs issued before the first slipped-in load
   static_assert(TM == TN, "the MFMA schedule assumes a square wave tile");
-  auto fetch_one = [&](int n, int ks, uint8_t* buf) {
+  // global_load_lds_dwordx4 in its scalar-base + 32-bit-lane-offset form (the builtin is
+  // selected with a 64-bit address per lane, which costs a 64-bit add and a second address
+  // register per load); M0 carries the LDS destination.
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
+  auto dma16 = [&](const uint8_t* uniform_base, uint32_t lane_off, uint32_t lds_off) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_base + lds_off), "v"(lane_off), "s"(uniform_base)
+                 : "memory");  // M0 has no other user in this kernel (LDS reads do not need it on gfx9+)
+  };
+  auto fetch_one = [&](int n, int ks, uint32_t buf) {
     if (n < kLoadsA) {
-      __builtin_amdgcn_global_load_lds((gptr_t)(A + (int64_t)ks * kBK + offA[n]),
-                                       (lptr_t)(buf + (wave * kLoadsA + n) * kGroupStride), 16, 0, 0);
+      dma16(A + (int64_t)ks * kBK, offA[n], buf + (wave * kLoadsA + n) * kGroupStride);
     } else if (n < kLoadsA + kLoadsB) {
       const int i = n - kLoadsA;
-      __builtin_amdgcn_global_load_lds((gptr_t)(B + (int64_t)ks * kBK + offB[i]),
-                                       (lptr_t)(buf + kOffB + (wave * kLoadsB + i) * kGroupStride), 16, 0, 0);
+      dma16(B + (int64_t)ks * kBK, offB[i], buf + kOffB + (wave * kLoadsB + i) * kGroupStride);
     } else {
-      __builtin_amdgcn_global_load_lds((gptr_t)(sc_src + (int64_t)ks * 512), (lptr_t)(buf + sc_dst), 16, 0, 0);
+      dma16(sc_base + (int64_t)ks * 512, sc_off, buf + sc_dst);
     }
   };
-  auto fetch = [&](int ks, uint8_t* buf) {
+  auto fetch = [&](int ks, uint32_t buf) {
 #pragma unroll
     for (int n = 0; n < kLoadsPerStep; ++n) fetch_one(n, ks, buf);
   };
@@ -181,7 +187,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // prologue: steps 0 .. NST-2 into the first ring slots (clamped for very short K)
   constexpr int kAhead = NST - 1;  // steps in flight ahead of the one being multiplied
 #pragma unroll
-  for (int p = 0; p < kAhead; ++p) fetch(p < k_steps ? p : k_steps - 1, lds + p * kStageBytes);
+  for (int p = 0; p < kAhead; ++p) fetch(p < k_steps ? p : k_steps - 1, (uint32_t)(p * kStageBytes));
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kAhead - 1) * kLoadsPerStep) : "memory");
   __syncthreads();
 
@@ -193,7 +199,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     // compiler sinks the MFMAs below the wait and barrier, which serialises memory and math.
     const uint32_t cur = slot * kStageBytes;
     const int slot_load = slot == 0 ? NST - 1 : slot - 1;  // the slot read in the previous step
-    uint8_t* nxt = lds + slot_load * kStageBytes;
+    const uint32_t nxt = slot_load * kStageBytes;
     const int kn = ks + kAhead < k_steps ? ks + kAhead : k_steps - 1;
     slot = slot + 1 == NST ? 0 : slot + 1;
     __builtin_amdgcn_sched_barrier(0);
@@ -273,7 +279,7 @@ template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int FIRST, int EVER
 int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N,
                 int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream) {
   const int tiles_m = (int)ceil_div(M, BM), tiles_n = (int)ceil_div(N, BN);
-  size_t lds_bytes = (size_t)NST * (((BM + BN) / kGroupRows) * kGroupStride + ((BM + BN) / 128) * 512);  // NST K-steps
+  size_t lds_bytes = (size_t)NST * (((BM + BN) / kGroupRows) * kGroupStride + 2048);  // NST K-steps: panels + scale slots
   // A grid that fits the chip once should land one workgroup per CU: asking for more than half
   // of the LDS keeps the dispatcher from pairing two workgroups on one CU while others idle.
   if ((int64_t)tiles_m * tiles_n <= device_facts().cu_count && lds_bytes < 82 * 1024) lds_bytes = 82 * 1024;
