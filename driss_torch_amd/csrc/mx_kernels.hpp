@@ -270,10 +270,17 @@ __global__ __launch_bounds__(kBlock) void mx_col_t_kernel(const void* __restrict
   __shared__ __attribute__((aligned(16))) uint8_t tile[kColTCols * kColTPitch];
   __shared__ __attribute__((aligned(16))) uint32_t stile[kColTCols];  // 4 scale bytes per column
   const int tid = threadIdx.x, lane = tid % kWave, w = tid / kWave;
-  // consecutive workgroups walk down the rows, so their 128-byte output segments are adjacent
-  // (measured 7% faster than walking along the columns)
+  // Tiles are numbered down the rows first, so that neighbours write adjacent 128-byte output
+  // segments and adjacent words of the same scale line.  Workgroup b runs on XCD b % 8 and
+  // each XCD has its own L2: runs of 8 consecutive tiles are given to one XCD (workgroups
+  // b, b+8, ... which start together), so that its L2 can merge their partial lines.
   const uint32_t row_tiles128 = (rows + kColTRows - 1) / kColTRows;
-  const uint32_t tc = blockIdx.x / row_tiles128, tr = blockIdx.x - tc * row_tiles128;
+  uint32_t t = blockIdx.x;
+  if (t < (gridDim.x & ~63u)) {
+    const uint32_t xcd = t & 7u, slot = t >> 3;
+    t = (slot & ~7u) * 8u + xcd * 8u + (slot & 7u);
+  }
+  const uint32_t tc = t / row_tiles128, tr = t - tc * row_tiles128;
   const uint32_t row0 = tr * kColTRows + w * 32, col0 = tc * kColTCols + lane * 4;
   const bool active = row0 < rows && col0 < cols;  // rows % 32 == 0 and cols % 4 == 0
 
