@@ -36,7 +36,7 @@ constexpr int kGroupStride = 1024;   // 8 rows of 128 bytes; the chunk swizzle a
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int FIRST, int EVERY>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int MID>
 __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const uint8_t* __restrict__ sfa,
     const uint8_t* __restrict__ sfb, int M, int N, int K, int64_t lda, int64_t ldb, uint16_t* __restrict__ out,
@@ -106,7 +106,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   const int sc_dst = wave_is_b ? kOffSB : kOffSA;
   // load number n of a step: n < kLoadsA -> A group, < kLoadsA+kLoadsB -> B group, else scales
   constexpr int kLoadsPerStep = kLoadsA + kLoadsB + 1;
-  constexpr int kFirstLoadAfter = FIRST;  // MFMAs issued before the first slipped-in load
   static_assert(TM == TN, "the MFMA schedule assumes a square wave tile");
   // global_load_lds_dwordx4 in its scalar-base + 32-bit-lane-offset form (the builtin is
   // selected with a 64-bit address per lane, which costs a 64-bit add and a second address
@@ -142,11 +141,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // fragment of tile row `l16` of a 16-row tile starting at panel row `row0` (multiple of 16):
   // logical chunks kq (K = 16kq..) and 4+kq (K = 64+16kq..), which sit 64 bytes apart (xor 4)
   const int kq = lane >> 4, l16 = lane & 15;
-  const uint32_t frag_lane_off = (l16 >> 3) * kGroupStride + (l16 & 7) * 128 + ((kq ^ (l16 & 7)) << 4);
-  auto load_frag = [&](uint32_t panel_off, int row0) -> v8i {
-    const uint32_t o = panel_off + (row0 >> 3) * kGroupStride + frag_lane_off;
-    const u32x4 lo = *reinterpret_cast<const u32x4*>(lds + o);
-    const u32x4 hi = *reinterpret_cast<const u32x4*>(lds + (o ^ 64u));
+  const uint32_t frag_lo = (l16 >> 3) * kGroupStride + (l16 & 7) * 128 + ((kq ^ (l16 & 7)) << 4);
+  const uint32_t frag_hi = frag_lo ^ 64u;  // stage and panel offsets are multiples of 1024: the xor commutes with them
+  auto load_frag = [&](uint32_t stage_lo, uint32_t stage_hi, int panel_off, int row0) -> v8i {
+    // stage_lo/hi = stage offset + frag_lo/hi (one add each per K-step); the rest is an immediate
+    const int o = panel_off + (row0 >> 3) * kGroupStride;
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(lds + stage_lo + o);
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(lds + stage_hi + o);
     return v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
   };
   // Scales of a staged 512-byte chunk (128 rows): the word of row r sits at
@@ -174,79 +175,124 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   };
   static_assert((TM == 8 || TM == 4) && (TN == 8 || TN == 4), "wave tile is 128 or 64 rows/columns");
 
-  // prologue: steps 0 .. NST-2 into the first ring slots (clamped for very short K)
-  constexpr int kAhead = NST - 1;  // steps in flight ahead of the one being multiplied
+  // Software pipeline.  Ring slot s holds K-step ks with ks % NST == s.  Inside step ks the
+  // wave first issues the MFMAs of the leading MID x MID square while it pulls the remaining
+  // fragments out of the slot; once the last fragment is in registers nobody needs the slot any
+  // more, so the step's one barrier sits THERE, in the middle of the MFMA stream, together with
+  // the wait for step ks+1 to have landed.  Behind the barrier, under the remaining MFMAs, the
+  // wave reads the scales and the first fragments of step ks+1 and issues the global->LDS loads
+  // of step ks+NST into the slot just released.  The MFMA pipe therefore never drains at a
+  // barrier: the LDS round trip that follows it is covered by MFMAs already queued.  With one
+  // wave per SIMD nothing else would hide it.  sched_barrier pins the order (the compiler
+  // otherwise sinks MFMAs below waits and barriers, which serialises memory and math).
+  static_assert(NST >= 2 && MID >= 2 && MID < TM && MID + 2 >= TM, "pipeline shape");
 #pragma unroll
-  for (int p = 0; p < kAhead; ++p) fetch(p < k_steps ? p : k_steps - 1, (uint32_t)(p * kStageBytes));
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kAhead - 1) * kLoadsPerStep) : "memory");
+  for (int p = 0; p < NST; ++p) fetch(p < k_steps ? p : k_steps - 1, (uint32_t)(p * kStageBytes));
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 1) * kLoadsPerStep) : "memory");
   __syncthreads();
+  constexpr int a_row0_w = WM, b_row0_w = WN;
+  const int a_row0 = wm * a_row0_w, b_row0 = wn * b_row0_w;
+  const bool a_upper = (wm & 1) != 0, b_upper = (wn & 1) != 0;
+  // only the wave's first row differs between waves: fold it into the per-lane bases
+  const uint32_t lane_lo_a = frag_lo + (a_row0 >> 3) * kGroupStride, lane_hi_a = frag_hi + (a_row0 >> 3) * kGroupStride;
+  const uint32_t lane_lo_b = frag_lo + (b_row0 >> 3) * kGroupStride, lane_hi_b = frag_hi + (b_row0 >> 3) * kGroupStride;
+  v8i fa[TM], fb[TN];
+  int sa[TM], sb[TN];
+  ScaleWords swb = load_scales(kOffSB, b_row0 & ~127);
+  ScaleWords swa = load_scales(kOffSA, a_row0 & ~127);
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    fa[t] = load_frag(lane_lo_a, lane_hi_a, 0, t * 16);
+    fb[t] = load_frag(lane_lo_b, lane_hi_b, kOffB, t * 16);
+    sa[t] = scale_of(swa, t, TM, a_upper);
+    sb[t] = scale_of(swb, t, TN, b_upper);
+  }
 
   int slot = 0;  // ring slot of step ks
   for (int ks = 0; ks < k_steps; ++ks) {
-    // Multiply this step while the loads of step ks+NST-1 are issued (clamped at the end, where
-    // the extra loads land in an idle slot and are ignored), then wait for step ks+1 to have
-    // landed and for the other waves.  The scheduling fences pin the order: without them the
-    // compiler sinks the MFMAs below the wait and barrier, which serialises memory and math.
     const uint32_t cur = slot * kStageBytes;
-    const int slot_load = slot == 0 ? NST - 1 : slot - 1;  // the slot read in the previous step
-    const uint32_t nxt = slot_load * kStageBytes;
-    const int kn = ks + kAhead < k_steps ? ks + kAhead : k_steps - 1;
     slot = slot + 1 == NST ? 0 : slot + 1;
+    const uint32_t nxt = slot * kStageBytes;                           // step ks+1
+    const int kn = ks + NST < k_steps ? ks + NST : k_steps - 1;       // refill of `cur` (clamped at the end: ignored)
+    const uint32_t cla = cur + lane_lo_a, cha = cur + lane_hi_a, clb = cur + lane_lo_b, chb = cur + lane_hi_b;
     __builtin_amdgcn_sched_barrier(0);
-
-    v8i fb[TN];
-    const ScaleWords swb = load_scales(cur + kOffSB, (wn * WN) & ~127);
-    const ScaleWords swa = load_scales(cur + kOffSA, (wm * WM) & ~127);
-    // Expanding-square order: step k of the schedule loads fragments a[k+1], b[k+1] and issues
-    // the 2k+1 MFMAs that a[k], b[k] make possible, so the first MFMA waits for two fragments
-    // only and the LDS burst after the barrier overlaps with math.  With one wave per SIMD
-    // nothing else hides instruction issue, so the global->LDS loads of the step ahead are
-    // slipped in one at a time behind MFMAs (an MFMA keeps the pipe busy for 8 passes while
-    // the wave issues something else).  sched_barrier pins this order.
-    v8i fa[TM];
-    fa[0] = load_frag(cur, wm * WM);
-    fb[0] = load_frag(cur + kOffB, wn * WN);
-    if (TM > 1) {
-      fa[1] = load_frag(cur, wm * WM + 16);
-      fb[1] = load_frag(cur + kOffB, wn * WN + 16);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    int sa[TM], sb[TN];
-#pragma unroll
-    for (int t = 0; t < TM; ++t) sa[t] = scale_of(swa, t, TM, (wm & 1) != 0);
-#pragma unroll
-    for (int t = 0; t < TN; ++t) sb[t] = scale_of(swb, t, TN, (wn & 1) != 0);
-    __builtin_amdgcn_sched_barrier(0);
-    int n_load = 0, n_mfma = 0;
     auto mfma = [&](int i, int j) {
       // B fragment as the row operand: acc[i][j][v] = D[m = l16][n = 4*kq + v] of the tile
       acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], fa[i], acc[i][j], 0, 0, 0, sb[j], 0, sa[i]);
-      if (n_load < kLoadsPerStep && n_mfma >= kFirstLoadAfter && (n_mfma - kFirstLoadAfter) % EVERY == 0) {
-        fetch_one(n_load, kn, nxt);
-        ++n_load;
-      }
-      ++n_mfma;
-      __builtin_amdgcn_sched_barrier(0);
     };
+    // ---- before the barrier.  Expanding-square order: round k requests fragments a[k+2], b[k+2]
+    // (and shifts their scale bytes into place) and issues the 2k+1 MFMAs that a[k], b[k] make
+    // possible, so an MFMA never waits for more than two fragments.
 #pragma unroll
-    for (int k = 0; k < TM; ++k) {
+    for (int k = 0; k < MID; ++k) {
       if (k + 2 < TM) {
-        fa[k + 2] = load_frag(cur, wm * WM + (k + 2) * 16);
-        fb[k + 2] = load_frag(cur + kOffB, wn * WN + (k + 2) * 16);
+        fa[k + 2] = load_frag(cla, cha, 0, (k + 2) * 16);
+        fb[k + 2] = load_frag(clb, chb, kOffB, (k + 2) * 16);
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
-      for (int j = 0; j <= k; ++j) mfma(k, j);
+      for (int j = 0; j <= k; ++j) {
+        mfma(k, j);
+        if (j == 0 && k + 2 < TM) {
+          sa[k + 2] = scale_of(swa, k + 2, TM, a_upper);
+          sb[k + 2] = scale_of(swb, k + 2, TN, b_upper);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
 #pragma unroll
-      for (int i = 0; i < k; ++i) mfma(i, k);
+      for (int i = 0; i < k; ++i) {
+        mfma(i, k);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // every fragment of this step has been requested; once they are in, the slot is free
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_waitcnt vmcnt(%0)" ::"n"((NST - 2) * kLoadsPerStep) : "memory");
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- behind the barrier: rounds MID.., the MFMAs that read fragments 0 and 1 first, so that
+    // the first fragments of the next step can land in the same registers.  One item of other
+    // work follows each MFMA: the scale words of step ks+1, the refill of this slot, the
+    // fragments, and last the scale bytes of the first two tiles.
+    constexpr int kHead = 4 * (TM - MID);                      // MFMAs that still read fragments 0, 1
+    constexpr int kBehind = TM * TM - MID * MID;               // MFMAs behind the barrier
+    const uint32_t nla = nxt + lane_lo_a, nha = nxt + lane_hi_a, nlb = nxt + lane_lo_b, nhb = nxt + lane_hi_b;
+    int m = 0, n_dma = 0;
+    auto behind = [&](int i, int j) {
+      mfma(i, j);
+      if (m == 0) swb = load_scales(nxt + kOffSB, b_row0 & ~127);
+      else if (m == 1) swa = load_scales(nxt + kOffSA, a_row0 & ~127);
+      else if (m == kHead) fa[0] = load_frag(nla, nha, 0, 0);
+      else if (m == kHead + 1) fb[0] = load_frag(nlb, nhb, kOffB, 0);
+      else if (m == kHead + 2) fa[1] = load_frag(nla, nha, 0, 16);
+      else if (m == kHead + 3) fb[1] = load_frag(nlb, nhb, kOffB, 16);
+      else if (n_dma < kLoadsPerStep) fetch_one(n_dma++, kn, cur);
+      if (m == kBehind - 2) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          sa[t] = scale_of(swa, t, TM, a_upper);
+          sb[t] = scale_of(swb, t, TN, b_upper);
+        }
+      }
+      ++m;
+      __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int k = MID; k < TM; ++k) {
+      behind(k, 0); behind(k, 1); behind(0, k); behind(1, k);
     }
 #pragma unroll
-    for (; n_load < kLoadsPerStep; ++n_load) fetch_one(n_load, kn, nxt);
-    // the next step's panels must have landed (later ones may still be in flight), and every
-    // wave must be done reading `cur`
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kAhead - 1) * kLoadsPerStep) : "memory");
-    __syncthreads();
+    for (int k = MID; k < TM; ++k) {
+#pragma unroll
+      for (int j = 2; j <= k; ++j) behind(k, j);
+#pragma unroll
+      for (int i = 2; i < k; ++i) behind(i, k);
+    }
+#pragma unroll
+    for (; n_dma < kLoadsPerStep; ++n_dma) fetch_one(n_dma, kn, cur);
   }
+  // the clamped refills of the last steps may still be landing: the epilogue reuses the LDS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
 
   // ---- epilogue: fp32 -> bf16 (v_cvt_pk_bf16_f32, round to nearest even) and out through LDS.
   // A lane holds 4 consecutive columns of one row per tile; written straight to memory that is
@@ -285,7 +331,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int FIRST, int EVERY>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int MID>
 int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N,
                 int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream) {
   const int tiles_m = (int)ceil_div(M, BM), tiles_n = (int)ceil_div(N, BN);
@@ -295,7 +341,7 @@ int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const ui
   // A grid that fits the chip once should land one workgroup per CU: asking for more than half
   // of the LDS keeps the dispatcher from pairing two workgroups on one CU while others idle.
   if ((int64_t)tiles_m * tiles_n <= device_facts().cu_count && lds_bytes < 82 * 1024) lds_bytes = 82 * 1024;
-  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST, FIRST, EVERY>;
+  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST, MID>;
   if (lds_bytes > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess)
@@ -325,7 +371,7 @@ extern "C" int dt_mx_fp8_bf16(const void* a, const void* b, const uint8_t* sfa, 
   const int variant = dt::tuning("gemm.variant");
   const int64_t tiles256 = dt::ceil_div(M, 256) * dt::ceil_div(N, 256);
   const bool big = variant == 2 || (variant == 0 && tiles256 >= dt::device_facts().cu_count / 2);
-  // <tile M, tile N, waves M, waves N, LDS ring slots, first slipped-in load after MFMA #, one every # MFMAs>
-  if (big) return dt::launch_gemm<256, 256, 2, 2, 2, 0, 2>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
-  return dt::launch_gemm<128, 128, 2, 2, 4, 1, 2>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  // <tile M, tile N, waves M, waves N, LDS ring slots, MFMA round at which the step's barrier sits>
+  if (big) return dt::launch_gemm<256, 256, 2, 2, 2, 6>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  return dt::launch_gemm<128, 128, 2, 2, 4, 2>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
 }
