@@ -10,8 +10,8 @@
 // A workgroup of 4 waves owns a BM x BN output tile and walks K in steps of 128.  The A and B
 // panels of a step go from global memory straight into LDS (global_load_lds_dwordx4: lane L of
 // a wave deposits its 16 bytes at LDS base + 16 L, so one wave instruction fills 8 rows of
-// 128 bytes) and are double buffered with one barrier per step: while step k is multiplied out
-// of one buffer, step k+1 lands in the other.  Inside an 8-row group the 16-byte chunks of row
+// 128 bytes) into a ring of NST stages, with one barrier per step placed in the middle of the
+// step's MFMA stream (see the main loop).  Inside an 8-row group the 16-byte chunks of row
 // r sit at chunk ^ (r & 7), which makes the 16-byte fragment reads of 16 consecutive rows
 // conflict-free (measured: 6.25 clk per wave read, the same as a linear read; 144-byte padded
 // rows cost 8, unswizzled rows 16).  The step's E8M0 scale chunks of the blocked buffers
@@ -36,7 +36,7 @@ constexpr int kGroupStride = 1024;   // 8 rows of 128 bytes; the chunk swizzle a
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int MID>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST>
 __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const uint8_t* __restrict__ sfa,
     const uint8_t* __restrict__ sfb, int M, int N, int K, int64_t lda, int64_t ldb, uint16_t* __restrict__ out,
@@ -157,10 +157,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   struct ScaleWords {
     u32x4 even, odd;  // tiles 0,2,4,6 and 1,3,5,7 of a 128-row chunk
   };
-  auto load_scales = [&](uint32_t scale_off, int row0) -> ScaleWords {  // row0: multiple of 128
-    const uint32_t o = scale_off + (row0 >> 7) * 512 + l16 * 16;
-    return ScaleWords{*reinterpret_cast<const u32x4*>(lds + o), *reinterpret_cast<const u32x4*>(lds + o + 256)};
-  };
   // scale operand of wave tile t (compile-time) out of NT tiles; with 4 tiles per wave the wave
   // sits in the lower or upper half of its chunk
   const int scale_shift = kq * 8;
@@ -175,121 +171,127 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   };
   static_assert((TM == 8 || TM == 4) && (TN == 8 || TN == 4), "wave tile is 128 or 64 rows/columns");
 
-  // Software pipeline.  Ring slot s holds K-step ks with ks % NST == s.  Inside step ks the
-  // wave first issues the MFMAs of the leading MID x MID square while it pulls the remaining
-  // fragments out of the slot; once the last fragment is in registers nobody needs the slot any
-  // more, so the step's one barrier sits THERE, in the middle of the MFMA stream, together with
-  // the wait for step ks+1 to have landed.  Behind the barrier, under the remaining MFMAs, the
-  // wave reads the scales and the first fragments of step ks+1 and issues the global->LDS loads
-  // of step ks+NST into the slot just released.  The MFMA pipe therefore never drains at a
-  // barrier: the LDS round trip that follows it is covered by MFMAs already queued.  With one
-  // wave per SIMD nothing else would hide it.  sched_barrier pins the order (the compiler
-  // otherwise sinks MFMAs below waits and barriers, which serialises memory and math).
-  static_assert(NST >= 2 && MID >= 2 && MID < TM && MID + 2 >= TM, "pipeline shape");
+  // Software pipeline.  Ring slot s holds K-step ks with ks % NST == s.  The TM x TN grid of MFMAs
+  // of a step is cut into four quadrants over the fragment halves lo = [0, H) and hi = [H, 2H),
+  // issued in the order (a half, b half)
+  //                      (lo,hi) (lo,lo) | (hi,hi) (hi,lo)
+  // A step starts with a[lo] and b[hi] in registers.  During the first two quadrants it pulls
+  // b[lo] and a[hi] out of its slot; after them every fragment of the step is in registers,
+  // nobody needs the slot any more, and the step's one barrier sits THERE (the bar), in the
+  // middle of the MFMA stream, with the wait for step ks+1 to have landed.  Behind it a[lo] is
+  // dead, and after the third quadrant so is b[hi]: the wave reloads them with the fragments of
+  // step ks+1 and slips the global->LDS loads of step ks+NST into the slot just released.  So
+  // LDS reads are spread evenly over the step (one fragment per four MFMAs), every fragment is
+  // requested at least a quadrant before its first use, no register is needed twice, and the
+  // MFMA pipe never drains at the barrier.  With one wave per SIMD nothing else would hide those
+  // latencies.  sched_barrier pins the order (the compiler otherwise sinks MFMAs below waits and
+  // barriers).
+  static_assert(NST >= 2 && TM == TN && TM % 2 == 0, "pipeline shape");
+  constexpr int H = TM / 2;
+  constexpr std::integral_constant<int, 0> kLo{};
+  constexpr std::integral_constant<int, H> kHi{};
 #pragma unroll
   for (int p = 0; p < NST; ++p) fetch(p < k_steps ? p : k_steps - 1, (uint32_t)(p * kStageBytes));
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 1) * kLoadsPerStep) : "memory");
   __syncthreads();
-  constexpr int a_row0_w = WM, b_row0_w = WN;
-  const int a_row0 = wm * a_row0_w, b_row0 = wn * b_row0_w;
+  const int a_row0 = wm * WM, b_row0 = wn * WN;
   const bool a_upper = (wm & 1) != 0, b_upper = (wn & 1) != 0;
   // only the wave's first row differs between waves: fold it into the per-lane bases
   const uint32_t lane_lo_a = frag_lo + (a_row0 >> 3) * kGroupStride, lane_hi_a = frag_hi + (a_row0 >> 3) * kGroupStride;
   const uint32_t lane_lo_b = frag_lo + (b_row0 >> 3) * kGroupStride, lane_hi_b = frag_hi + (b_row0 >> 3) * kGroupStride;
+  const uint32_t sc_lane_a = ((a_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSA;
+  const uint32_t sc_lane_b = ((b_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSB;
+  auto read_scales = [&](uint32_t o) -> ScaleWords {
+    return ScaleWords{*reinterpret_cast<const u32x4*>(lds + o), *reinterpret_cast<const u32x4*>(lds + o + 256)};
+  };
   v8i fa[TM], fb[TN];
   int sa[TM], sb[TN];
-  ScaleWords swb = load_scales(kOffSB, b_row0 & ~127);
-  ScaleWords swa = load_scales(kOffSA, a_row0 & ~127);
+  ScaleWords swa = read_scales(sc_lane_a), swb = read_scales(sc_lane_b);
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
+  for (int t = 0; t < H; ++t) {
     fa[t] = load_frag(lane_lo_a, lane_hi_a, 0, t * 16);
-    fb[t] = load_frag(lane_lo_b, lane_hi_b, kOffB, t * 16);
+    fb[H + t] = load_frag(lane_lo_b, lane_hi_b, kOffB, (H + t) * 16);
     sa[t] = scale_of(swa, t, TM, a_upper);
-    sb[t] = scale_of(swb, t, TN, b_upper);
+    sb[H + t] = scale_of(swb, H + t, TN, b_upper);
   }
 
   int slot = 0;  // ring slot of step ks
-  for (int ks = 0; ks < k_steps; ++ks) {
+  int ks = 0;
+  do {  // k_steps >= 1
     const uint32_t cur = slot * kStageBytes;
     slot = slot + 1 == NST ? 0 : slot + 1;
     const uint32_t nxt = slot * kStageBytes;                           // step ks+1
     const int kn = ks + NST < k_steps ? ks + NST : k_steps - 1;       // refill of `cur` (clamped at the end: ignored)
     const uint32_t cla = cur + lane_lo_a, cha = cur + lane_hi_a, clb = cur + lane_lo_b, chb = cur + lane_hi_b;
+    const uint32_t nla = nxt + lane_lo_a, nha = nxt + lane_hi_a, nlb = nxt + lane_lo_b, nhb = nxt + lane_hi_b;
+    int n_dma = 0;
     __builtin_amdgcn_sched_barrier(0);
-    auto mfma = [&](int i, int j) {
-      // B fragment as the row operand: acc[i][j][v] = D[m = l16][n = 4*kq + v] of the tile
-      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], fa[i], acc[i][j], 0, 0, 0, sb[j], 0, sa[i]);
+    // H*H MFMAs over a tiles i0.., b tiles j0.. with the b tile as the outer index (the b half
+    // of a step's first quadrant is the one requested last); `after(q)` follows MFMA number q
+    auto quadrant = [&](auto i0_tag, auto j0_tag, auto&& after) {
+      constexpr int i0 = decltype(i0_tag)::value, j0 = decltype(j0_tag)::value;
+#pragma unroll
+      for (int q = 0; q < H * H; ++q) {
+        const int i = i0 + q % H, j = j0 + q / H;
+        // B fragment as the row operand: acc[i][j][v] = D[m = l16][n = 4*kq + v] of the tile
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], fa[i], acc[i][j], 0, 0, 0, sb[j], 0, sa[i]);
+        after(q);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     };
-    // ---- before the barrier.  Expanding-square order: round k requests fragments a[k+2], b[k+2]
-    // (and shifts their scale bytes into place) and issues the 2k+1 MFMAs that a[k], b[k] make
-    // possible, so an MFMA never waits for more than two fragments.
-#pragma unroll
-    for (int k = 0; k < MID; ++k) {
-      if (k + 2 < TM) {
-        fa[k + 2] = load_frag(cla, cha, 0, (k + 2) * 16);
-        fb[k + 2] = load_frag(clb, chb, kOffB, (k + 2) * 16);
-        __builtin_amdgcn_sched_barrier(0);
+    auto dma = [&]() {
+      if (n_dma < kLoadsPerStep) fetch_one(n_dma++, kn, cur);
+    };
+    // ---- before the bar: (lo,hi) pulls b[lo], (lo,lo) pulls a[hi]
+    quadrant(kLo, kHi, [&](int q) {
+      if (q % H == 0) {
+        const int t = q / H;
+        fb[t] = load_frag(clb, chb, kOffB, t * 16);
+        sb[t] = scale_of(swb, t, TN, b_upper);
       }
-#pragma unroll
-      for (int j = 0; j <= k; ++j) {
-        mfma(k, j);
-        if (j == 0 && k + 2 < TM) {
-          sa[k + 2] = scale_of(swa, k + 2, TM, a_upper);
-          sb[k + 2] = scale_of(swb, k + 2, TN, b_upper);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+    });
+    quadrant(kLo, kLo, [&](int q) {
+      if (q % (H - 1) == 0 && q / (H - 1) < H) {
+        const int t = H + q / (H - 1);
+        fa[t] = load_frag(cla, cha, 0, t * 16);
+        sa[t] = scale_of(swa, t, TM, a_upper);
       }
-#pragma unroll
-      for (int i = 0; i < k; ++i) {
-        mfma(i, k);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
+    });
     // every fragment of this step has been requested; once they are in, the slot is free
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_waitcnt vmcnt(%0)" ::"n"((NST - 2) * kLoadsPerStep) : "memory");
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
-    // ---- behind the barrier: rounds MID.., the MFMAs that read fragments 0 and 1 first, so that
-    // the first fragments of the next step can land in the same registers.  One item of other
-    // work follows each MFMA: the scale words of step ks+1, the refill of this slot, the
-    // fragments, and last the scale bytes of the first two tiles.
-    constexpr int kHead = 4 * (TM - MID);                      // MFMAs that still read fragments 0, 1
-    constexpr int kBehind = TM * TM - MID * MID;               // MFMAs behind the barrier
-    const uint32_t nla = nxt + lane_lo_a, nha = nxt + lane_hi_a, nlb = nxt + lane_lo_b, nhb = nxt + lane_hi_b;
-    int m = 0, n_dma = 0;
-    auto behind = [&](int i, int j) {
-      mfma(i, j);
-      if (m == 0) swb = load_scales(nxt + kOffSB, b_row0 & ~127);
-      else if (m == 1) swa = load_scales(nxt + kOffSA, a_row0 & ~127);
-      else if (m == kHead) fa[0] = load_frag(nla, nha, 0, 0);
-      else if (m == kHead + 1) fb[0] = load_frag(nlb, nhb, kOffB, 0);
-      else if (m == kHead + 2) fa[1] = load_frag(nla, nha, 0, 16);
-      else if (m == kHead + 3) fb[1] = load_frag(nlb, nhb, kOffB, 16);
-      else if (n_dma < kLoadsPerStep) fetch_one(n_dma++, kn, cur);
-      if (m == kBehind - 2) {
+    // ---- behind the bar: (hi,hi) reloads a[lo], (hi,lo) reloads b[hi], both from step ks+1
+    constexpr int kFirstFrag = H > 2 ? 2 : 1, kFragEvery = H > 2 ? 3 : 1;
+    quadrant(kHi, kHi, [&](int q) {
+      if (q == 0) swb = read_scales(nxt + sc_lane_b);
+      if (q == (H > 2 ? 1 : 0)) swa = read_scales(nxt + sc_lane_a);
+      const int f = (q - kFirstFrag) / kFragEvery;
+      if (q >= kFirstFrag && (q - kFirstFrag) % kFragEvery == 0 && f < H) fa[f] = load_frag(nla, nha, 0, f * 16);
+      else if (q >= 2 || H == 2) dma();
+      if (q == H * H - 1) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          sa[t] = scale_of(swa, t, TM, a_upper);
-          sb[t] = scale_of(swb, t, TN, b_upper);
-        }
+        for (int t = 0; t < H; ++t) sa[t] = scale_of(swa, t, TM, a_upper);
       }
-      ++m;
-      __builtin_amdgcn_sched_barrier(0);
-    };
+    });
 #pragma unroll
-    for (int k = MID; k < TM; ++k) {
-      behind(k, 0); behind(k, 1); behind(0, k); behind(1, k);
-    }
+    for (int t = 0; t < kLoadsPerStep / 2; ++t)
+      if (n_dma < kLoadsPerStep / 2) dma();
+    quadrant(kHi, kLo, [&](int q) {
+      if (q % H == 0) {
+        const int t = H + q / H;
+        fb[t] = load_frag(nlb, nhb, kOffB, t * 16);
+      } else {
+        dma();
+      }
+      if (q == H * H - 1) {
 #pragma unroll
-    for (int k = MID; k < TM; ++k) {
+        for (int t = 0; t < H; ++t) sb[H + t] = scale_of(swb, H + t, TN, b_upper);
+      }
+    });
 #pragma unroll
-      for (int j = 2; j <= k; ++j) behind(k, j);
-#pragma unroll
-      for (int i = 2; i < k; ++i) behind(i, k);
-    }
-#pragma unroll
-    for (; n_dma < kLoadsPerStep; ++n_dma) fetch_one(n_dma, kn, cur);
-  }
+    for (int t = 0; t < kLoadsPerStep; ++t) dma();
+  } while (++ks < k_steps);
   // the clamped refills of the last steps may still be landing: the epilogue reuses the LDS
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
@@ -331,7 +333,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, int MID>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST>
 int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N,
                 int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream) {
   const int tiles_m = (int)ceil_div(M, BM), tiles_n = (int)ceil_div(N, BN);
@@ -341,7 +343,7 @@ int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const ui
   // A grid that fits the chip once should land one workgroup per CU: asking for more than half
   // of the LDS keeps the dispatcher from pairing two workgroups on one CU while others idle.
   if ((int64_t)tiles_m * tiles_n <= device_facts().cu_count && lds_bytes < 82 * 1024) lds_bytes = 82 * 1024;
-  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST, MID>;
+  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST>;
   if (lds_bytes > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess)
@@ -371,7 +373,7 @@ extern "C" int dt_mx_fp8_bf16(const void* a, const void* b, const uint8_t* sfa, 
   const int variant = dt::tuning("gemm.variant");
   const int64_t tiles256 = dt::ceil_div(M, 256) * dt::ceil_div(N, 256);
   const bool big = variant == 2 || (variant == 0 && tiles256 >= dt::device_facts().cu_count / 2);
-  // <tile M, tile N, waves M, waves N, LDS ring slots, MFMA round at which the step's barrier sits>
-  if (big) return dt::launch_gemm<256, 256, 2, 2, 2, 6>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
-  return dt::launch_gemm<128, 128, 2, 2, 4, 2>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  // <tile M, tile N, waves M, waves N, LDS ring slots>
+  if (big) return dt::launch_gemm<256, 256, 2, 2, 2>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  return dt::launch_gemm<128, 128, 2, 2, 4>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
 }
