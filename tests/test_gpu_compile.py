@@ -1,0 +1,85 @@
+"""torch.compile coverage of every op of the path: each wrapper traced with fullgraph=True (so the
+fake implementations must produce the right shapes, dtypes and strides) and run through a backend
+that needs no code generator, compared bit for bit with the direct call.  Follows
+test/test_sat_cast.py:45-62, which does this for saturated_cast only."""
+import pytest
+import torch
+
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+
+
+@pytest.fixture(scope="module")
+def d(gpu_device):
+    import driss_torch_amd
+
+    return driss_torch_amd
+
+
+def _compiled(fn):
+    torch._dynamo.reset()
+    return torch.compile(fn, fullgraph=True, backend="aot_eager")
+
+
+def _same(a, b):
+    if isinstance(a, (tuple, list)):
+        assert len(a) == len(b)
+        for x, y in zip(a, b):
+            _same(x, y)
+        return
+    assert a.dtype == b.dtype and a.shape == b.shape and a.stride() == b.stride()
+    if a.dtype in (E4, E5, torch.float8_e8m0fnu):
+        assert torch.equal(util.codes(a), util.codes(b))
+    else:
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_amax_compile(d, dtype):
+    x = util.normal((256, 1024), 7001, dtype).cuda()
+    _same(_compiled(d.amax)(x), d.amax(x))
+
+
+@pytest.mark.parametrize("fp8_dtype", [E4, E5])
+def test_dynamic_scaled_quant_compile(d, fp8_dtype):
+    x = util.normal((512, 1024), 7002).cuda()
+    _same(_compiled(d.dynamic_scaled_quant)(x, fp8_dtype), d.dynamic_scaled_quant(x, fp8_dtype))
+    _same(_compiled(d.dynamic_scaled_quant_ex)(x, fp8_dtype), d.dynamic_scaled_quant_ex(x, fp8_dtype))
+    _same(_compiled(d.dynamic_scaled_quant_rowwise)(x, fp8_dtype), d.dynamic_scaled_quant_rowwise(x, fp8_dtype))
+
+
+def test_dynamic_scaled_quant_pair_compile(d):
+    x = util.normal((512, 1024), 7003).cuda()
+    _same(_compiled(d.dynamic_scaled_quant_pair)(x), d.dynamic_scaled_quant_pair(x))
+
+
+@pytest.mark.parametrize("axis,transpose", [(1, False), (0, False), (0, True), (1, True)])
+def test_mx_fp8_quantize_compile(d, axis, transpose):
+    x = util.normal((256, 512), 7004).cuda()
+
+    def fn(t):
+        return d.mx_fp8_quantize(t, 32, axis, transpose, E4)
+
+    _same(_compiled(fn)(x), fn(x))
+
+
+def test_mx_quantize_blocked_and_gemm_compile(d):
+    a = util.normal((256, 512), 7005).cuda()
+    b = util.normal((384, 512), 7006).cuda()
+
+    def fn(a, b):
+        ad, sa = d.mx_fp8_quantize_blocked(a)
+        bd, sb = d.mx_fp8_quantize_blocked(b)
+        return d.mx_fp8_bf16(ad, bd.t(), sa, sb)
+
+    got, want = _compiled(fn)(a, b), fn(a, b)
+    assert got.shape == (256, 384) and got.dtype == torch.bfloat16
+    _same(got, want)
+
+
+def test_to_blocked_compile(d):
+    s = torch.randint(0, 255, (256, 12), dtype=torch.uint8, device="cuda")
+    _same(_compiled(d.to_blocked)(s), d.to_blocked(s))
