@@ -86,7 +86,12 @@ def mx_fp8_bf16(a: Tensor, b: Tensor, a_scale: Tensor, b_scale: Tensor) -> Tenso
 
 
 def mx_fp4_bf16(a: Tensor, b: Tensor, a_scale: Tensor, b_scale: Tensor) -> Tensor:
-    """Schema kept from the reference (driss_torch/__init__.py:97-111); not built, raises."""
+    """bf16 = (a * 2^a_scale) @ (b * 2^b_scale) for e2m1 operands with E8M0 block-32 scales in
+    the blocked 128x4 layout (reference: driss_torch/__init__.py:97-111).
+
+    a: [M, K/2] row-major, b: [K/2, N] with stride(0) == 1; two e2m1 values per byte (uint8 or
+    float4_e2m1fn_x2 storage), the even element in the low nibble.
+    """
     return ops.mx_fp4_bf16(a, b, a_scale, b_scale)
 
 

@@ -83,3 +83,8 @@ def to_blocked_meta(scale):
 @register_fake("DrissTorch::mx_fp8_bf16")
 def mx_fp8_bf16_meta(a, b, a_scale, b_scale):
     return torch.empty((a.shape[0], b.shape[1]), dtype=torch.bfloat16, device=a.device)
+
+
+@register_fake("DrissTorch::mx_fp4_bf16")
+def mx_fp4_bf16_meta(a, b, a_scale, b_scale):
+    return torch.empty((a.shape[0], b.shape[1]), dtype=torch.bfloat16, device=a.device)

@@ -40,6 +40,7 @@ SIGNATURES = {
     "dt_blocked_scale_bytes": (_i64, [_i64, _i64]),
     "dt_to_blocked": (_i32, [_vp, _i64, _i64, _vp, _vp]),
     "dt_mx_fp8_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
+    "dt_mx_fp4_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     "dt_set_tuning": (_i32, [_cp, _i32]),
     "dt_get_tuning": (_i32, [_cp, C.POINTER(_i32)]),
 }
@@ -210,4 +211,14 @@ def mx_fp8_bf16(a: torch.Tensor, bt: torch.Tensor, sfa: torch.Tensor, sfb: torch
     out = torch.empty((M, N), dtype=torch.bfloat16, device=a.device) if out is None else out
     _check(lib().dt_mx_fp8_bf16(a.data_ptr(), bt.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), M, N, K, a.stride(0),
                                 bt.stride(0), out.data_ptr(), out.stride(0), _stream()), "dt_mx_fp8_bf16")
+    return out
+
+
+def mx_fp4_bf16(a: torch.Tensor, bt: torch.Tensor, sfa: torch.Tensor, sfb: torch.Tensor, out=None) -> torch.Tensor:
+    """a [M,K/2], bt [N,K/2] packed e2m1 pairs (both K-contiguous), blocked scales -> bf16 [M,N]."""
+    M, Kp = a.shape
+    N = bt.shape[0]
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=a.device) if out is None else out
+    _check(lib().dt_mx_fp4_bf16(a.data_ptr(), bt.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), M, N, 2 * Kp, a.stride(0),
+                                bt.stride(0), out.data_ptr(), out.stride(0), _stream()), "dt_mx_fp4_bf16")
     return out

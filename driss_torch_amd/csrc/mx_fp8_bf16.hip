@@ -27,6 +27,7 @@
 namespace dt {
 
 typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kBK = 128;             // K bytes per step = one 16x16x128 MFMA
@@ -36,7 +37,13 @@ constexpr int kGroupStride = 1024;   // 8 rows of 128 bytes; the chunk swizzle a
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST>
+// FP4: both operands are e2m1 nibbles, two per byte with the even element in the low nibble
+// (measured on gfx950: with format 4 lane 16g+i supplies row i, K = 32g..32g+31 in its first
+// four VGPRs, element k in nibble k%8 of word (k%32)/8).  A 128-byte LDS row then holds 256
+// elements = two MFMAs: bytes 16g.. of the first half feed the first, bytes 64+16g.. the second,
+// which are the same two 16-byte reads a lane makes for e4m3.  Everything else (panels, DMA,
+// swizzle, ring, quadrant schedule, epilogue) is shared; a K-step carries twice the scales.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4>
 __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const uint8_t* __restrict__ sfa,
     const uint8_t* __restrict__ sfb, int M, int N, int K, int64_t lda, int64_t ldb, uint16_t* __restrict__ out,
@@ -44,11 +51,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   constexpr int kThreads = WAVES_M * WAVES_N * kWave;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
   constexpr int TM = WM / 16, TN = WN / 16;            // MFMA tiles per wave
+  constexpr int KC = FP4 ? 2 : 1;                      // 128-element MFMAs (and blocked scale chunks) per K-step
 
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int kGroupsA = BM / kGroupRows, kGroupsB = BN / kGroupRows;
   constexpr int kPanelA = kGroupsA * kGroupStride, kPanelB = kGroupsB * kGroupStride;
-  constexpr int kScaleA = 1024, kScaleB = 1024;  // up to two 512-byte blocked scale chunks of one K-step each
+  constexpr int kScaleA = 1024 * KC, kScaleB = 1024 * KC;  // per chunk of the K-step: two 512-byte blocked scale chunks (2 x 128 rows)
   constexpr int kOffB = kPanelA, kOffSA = kPanelA + kPanelB, kOffSB = kOffSA + kScaleA;
   constexpr int kStageBytes = kOffSB + kScaleB;  // one K-step: A panel, B panel, A scales, B scales
   constexpr int kWaves = WAVES_M * WAVES_N;
@@ -72,14 +80,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   const int tile_m = first_m + (bid % group_size) % gm;
   const int tile_n = (bid % group_size) / gm;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int k_steps = K / kBK;
+  // K counts elements; a row holds k_bytes bytes, a K-step is 128 of them.  With FP4 the last
+  // step may be half filled (K % 256 == 128): its second MFMA is then switched off through the
+  // scales (see scale_bits) and its loads stay inside the first 64 bytes.
+  const int k_bytes = FP4 ? K / 2 : K;
+  const int k_steps = (k_bytes + kBK - 1) / kBK;
+  const int k_chunks = K / 128;                                   // blocked scale chunks per 128 rows
+  const int half_step = (FP4 && (k_bytes % kBK) != 0) ? k_steps - 1 : -1;  // index of a half-filled step
 
   // ---- global -> LDS.  Wave w owns groups w*kLoads .. of each panel; lane L fills row L/8,
   // chunk position L%8 of the group, i.e. it fetches logical chunk (L%8) ^ (L/8) of that row.
-  // Rows past the edge re-read the last row; their products are never stored.  Wave 0 also
-  // brings the A scales of the step (one 512-byte chunk of the blocked buffer per 128 rows,
-  // 32 lanes x 16 bytes each), wave 1 the B scales.
+  // Rows past the edge re-read the last row; their products are never stored.
   const int lrow = lane >> 3, lchunk = (lane & 7) ^ lrow;
+  const uint32_t half_adj = (lchunk & 4) ? 64u : 0u;  // in a half-filled step chunks 4-7 re-read chunks 0-3
   uint32_t offA[kLoadsA], offB[kLoadsB];
 #pragma unroll
   for (int i = 0; i < kLoadsA; ++i) {
@@ -93,19 +106,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     gr = gr < N ? gr : N - 1;
     offB[i] = (uint32_t)((int64_t)gr * ldb + lchunk * 16);
   }
-  // Scales: one more wave-wide load per step.  Even waves bring A chunks, odd waves B chunks:
+  // Scales: KC more wave-wide loads per step.  Even waves bring A chunks, odd waves B chunks:
   // lanes 0-31 the tile's first 128-row chunk, lanes 32-63 the next one (the second chunk of a
   // 256-row tile; for a 128-row tile it lands in an unused half of the slot).  Every wave issues
-  // it (duplicates write identical bytes), which keeps the instruction stream free of branches.
+  // them (duplicates write identical bytes), which keeps the instruction stream free of branches.
   const bool wave_is_b = (wave & 1) != 0;
   const int chunk_max = (wave_is_b ? (N + 127) / 128 : (M + 127) / 128) - 1;
   int chunk = (wave_is_b ? n0 : m0) / 128 + (lane >> 5);
   chunk = chunk < chunk_max ? chunk : chunk_max;
   const uint8_t* sc_base = wave_is_b ? sfb : sfa;
-  const uint32_t sc_off = (uint32_t)((int64_t)chunk * k_steps * 512 + (lane & 31) * 16);
+  const uint32_t sc_off = (uint32_t)((int64_t)chunk * k_chunks * 512 + (lane & 31) * 16);
   const int sc_dst = wave_is_b ? kOffSB : kOffSA;
   // load number n of a step: n < kLoadsA -> A group, < kLoadsA+kLoadsB -> B group, else scales
-  constexpr int kLoadsPerStep = kLoadsA + kLoadsB + 1;
+  constexpr int kLoadsPerStep = kLoadsA + kLoadsB + KC;
   static_assert(TM == TN, "the MFMA schedule assumes a square wave tile");
   // global_load_lds_dwordx4 in its scalar-base + 32-bit-lane-offset form (the builtin is
   // selected with a 64-bit address per lane, which costs a 64-bit add and a second address
@@ -118,13 +131,17 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
                  : "memory");  // M0 has no other user in this kernel (LDS reads do not need it on gfx9+)
   };
   auto fetch_one = [&](int n, int ks, uint32_t buf) {
+    const uint32_t adj = (FP4 && ks == half_step) ? half_adj : 0u;
     if (n < kLoadsA) {
-      dma16(A + (int64_t)ks * kBK, offA[n], buf + (wave * kLoadsA + n) * kGroupStride);
+      dma16(A + (int64_t)ks * kBK, offA[n] - adj, buf + (wave * kLoadsA + n) * kGroupStride);
     } else if (n < kLoadsA + kLoadsB) {
       const int i = n - kLoadsA;
-      dma16(B + (int64_t)ks * kBK, offB[i], buf + kOffB + (wave * kLoadsB + i) * kGroupStride);
+      dma16(B + (int64_t)ks * kBK, offB[i] - adj, buf + kOffB + (wave * kLoadsB + i) * kGroupStride);
     } else {
-      dma16(sc_base + (int64_t)ks * 512, sc_off, buf + sc_dst);
+      const int c = n - kLoadsA - kLoadsB;  // chunk of the step; past the end it re-reads the last one (switched off)
+      int kc = ks * KC + c;
+      kc = kc < k_chunks ? kc : k_chunks - 1;
+      dma16(sc_base + (int64_t)kc * 512, sc_off, buf + sc_dst + c * 1024);
     }
   };
   auto fetch = [&](int ks, uint32_t buf) {
@@ -139,35 +156,51 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
   // fragment of tile row `l16` of a 16-row tile starting at panel row `row0` (multiple of 16):
-  // logical chunks kq (K = 16kq..) and 4+kq (K = 64+16kq..), which sit 64 bytes apart (xor 4)
+  // logical chunks kq and 4+kq of the row, which sit 64 bytes apart (xor 4).  e4m3: K = 16kq..
+  // and 64+16kq.. of one MFMA; e2m1: K = 32kq.. of the step's first and of its second MFMA.
+  struct Frag {
+    v4i lo, hi;
+  };
   const int kq = lane >> 4, l16 = lane & 15;
   const uint32_t frag_lo = (l16 >> 3) * kGroupStride + (l16 & 7) * 128 + ((kq ^ (l16 & 7)) << 4);
   const uint32_t frag_hi = frag_lo ^ 64u;  // stage and panel offsets are multiples of 1024: the xor commutes with them
-  auto load_frag = [&](uint32_t stage_lo, uint32_t stage_hi, int panel_off, int row0) -> v8i {
+  auto load_frag = [&](uint32_t stage_lo, uint32_t stage_hi, int panel_off, int row0) -> Frag {
     // stage_lo/hi = stage offset + frag_lo/hi (one add each per K-step); the rest is an immediate
     const int o = panel_off + (row0 >> 3) * kGroupStride;
-    const u32x4 lo = *reinterpret_cast<const u32x4*>(lds + stage_lo + o);
-    const u32x4 hi = *reinterpret_cast<const u32x4*>(lds + stage_hi + o);
-    return v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    return Frag{*reinterpret_cast<const v4i*>(lds + stage_lo + o), *reinterpret_cast<const v4i*>(lds + stage_hi + o)};
   };
   // Scales of a staged 512-byte chunk (128 rows): the word of row r sits at
   // (r%32)*16 + (r/32)*4, so the 16 bytes at (r%32)*16 hold the words of rows r%32 + {0,32,64,96},
-  // i.e. of the four 16-row tiles t with the same parity.  Two reads per chunk cover its 8 tiles.
-  // A word holds the 4 K-block bytes of a row; the lane's own (K-block lane/16) goes to byte 0.
-  struct ScaleWords {
-    u32x4 even, odd;  // tiles 0,2,4,6 and 1,3,5,7 of a 128-row chunk
+  // i.e. of the four 16-row tiles t with the same parity (even tiles at l16*16, odd tiles 256
+  // bytes on).  A half of the wave tile (H tiles) is 8 or 4 bytes of each group.  A word holds
+  // the 4 K-block bytes of a row; the lane's own (K-block lane/16) goes to byte 0.
+  constexpr int H = TM / 2;
+  struct HalfWords {
+    uint32_t w[KC][H];  // [chunk of the step][tile of the half]
   };
-  // scale operand of wave tile t (compile-time) out of NT tiles; with 4 tiles per wave the wave
-  // sits in the lower or upper half of its chunk
-  const int scale_shift = kq * 8;
-  auto scale_of = [&](const ScaleWords& w, int t, int nt, bool upper) -> int {
-    auto word = [&](int tile) -> uint32_t {
-      const u32x4& v = (tile & 1) ? w.odd : w.even;
-      const int e = tile >> 1;
-      return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w;
-    };
-    const uint32_t x = nt == 8 ? word(t) : (upper ? word(4 + t) : word(t));
-    return (int)(x >> scale_shift);
+  auto read_half_scales = [&](uint32_t o, int half) -> HalfWords {  // o: stage + operand slot + lane part
+    HalfWords r;
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      if constexpr (H == 4) {
+        const u32x2 e = *reinterpret_cast<const u32x2*>(lds + o + c * 1024 + half * 8);
+        const u32x2 d = *reinterpret_cast<const u32x2*>(lds + o + c * 1024 + 256 + half * 8);
+        r.w[c][0] = e.x; r.w[c][1] = d.x; r.w[c][2] = e.y; r.w[c][3] = d.y;
+      } else {
+        r.w[c][0] = *reinterpret_cast<const uint32_t*>(lds + o + c * 1024 + half * 4);
+        r.w[c][1] = *reinterpret_cast<const uint32_t*>(lds + o + c * 1024 + 256 + half * 4);
+      }
+    }
+    return r;
+  };
+  // The scale operand: the lane's byte moved to bits 0-7.  For the second chunk of a half-filled
+  // step the field width is 0, so the byte reads as 0 = 2^-127: the MFMA's sum is scaled by
+  // 2^-254, underflows to zero (e2m1 has neither infinities nor NaNs) and leaves the accumulator
+  // as it is.
+  const uint32_t scale_shift = kq * 8;
+  auto scale_bits = [&](uint32_t word, int c, int step) -> int {
+    if (FP4 && c == 1) return (int)__builtin_amdgcn_ubfe(word, scale_shift, step == half_step ? 0u : 8u);
+    return (int)(word >> scale_shift);
   };
   static_assert((TM == 8 || TM == 4) && (TN == 8 || TN == 4), "wave tile is 128 or 64 rows/columns");
 
@@ -180,14 +213,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // nobody needs the slot any more, and the step's one barrier sits THERE (the bar), in the
   // middle of the MFMA stream, with the wait for step ks+1 to have landed.  Behind it a[lo] is
   // dead, and after the third quadrant so is b[hi]: the wave reloads them with the fragments of
-  // step ks+1 and slips the global->LDS loads of step ks+NST into the slot just released.  So
-  // LDS reads are spread evenly over the step (one fragment per four MFMAs), every fragment is
-  // requested at least a quadrant before its first use, no register is needed twice, and the
-  // MFMA pipe never drains at the barrier.  With one wave per SIMD nothing else would hide those
-  // latencies.  sched_barrier pins the order (the compiler otherwise sinks MFMAs below waits and
-  // barriers).
+  // step ks+1 and slips the global->LDS loads of step ks+NST into the slot just released.  The
+  // scale words of a half travel with its fragments: read at the start of a quadrant, shifted
+  // into place at its end.  So LDS reads are spread evenly over the step (one fragment per four
+  // MFMAs), every fragment is requested at least a quadrant before its first use, no register
+  // is needed twice, and the MFMA pipe never drains at the barrier.  With one wave per SIMD
+  // nothing else would hide those latencies.  sched_barrier pins the order (the compiler
+  // otherwise sinks MFMAs below waits and barriers).
   static_assert(NST >= 2 && TM == TN && TM % 2 == 0, "pipeline shape");
-  constexpr int H = TM / 2;
   constexpr std::integral_constant<int, 0> kLo{};
   constexpr std::integral_constant<int, H> kHi{};
 #pragma unroll
@@ -195,24 +228,26 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 1) * kLoadsPerStep) : "memory");
   __syncthreads();
   const int a_row0 = wm * WM, b_row0 = wn * WN;
-  const bool a_upper = (wm & 1) != 0, b_upper = (wn & 1) != 0;
   // only the wave's first row differs between waves: fold it into the per-lane bases
   const uint32_t lane_lo_a = frag_lo + (a_row0 >> 3) * kGroupStride, lane_hi_a = frag_hi + (a_row0 >> 3) * kGroupStride;
   const uint32_t lane_lo_b = frag_lo + (b_row0 >> 3) * kGroupStride, lane_hi_b = frag_hi + (b_row0 >> 3) * kGroupStride;
-  const uint32_t sc_lane_a = ((a_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSA;
-  const uint32_t sc_lane_b = ((b_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSB;
-  auto read_scales = [&](uint32_t o) -> ScaleWords {
-    return ScaleWords{*reinterpret_cast<const u32x4*>(lds + o), *reinterpret_cast<const u32x4*>(lds + o + 256)};
-  };
-  v8i fa[TM], fb[TN];
-  int sa[TM], sb[TN];
-  ScaleWords swa = read_scales(sc_lane_a), swb = read_scales(sc_lane_b);
+  // with 4 tiles per wave the wave sits in the lower or upper 8 bytes of the 16-byte scale groups
+  const uint32_t sc_lane_a = ((a_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSA + ((TM == 4 && (wm & 1)) ? 8 : 0);
+  const uint32_t sc_lane_b = ((b_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSB + ((TN == 4 && (wn & 1)) ? 8 : 0);
+  Frag fa[TM], fb[TN];
+  int sa[KC][TM], sb[KC][TN];
+  {
+    const HalfWords wa = read_half_scales(sc_lane_a, 0), wb = read_half_scales(sc_lane_b, 1);
 #pragma unroll
-  for (int t = 0; t < H; ++t) {
-    fa[t] = load_frag(lane_lo_a, lane_hi_a, 0, t * 16);
-    fb[H + t] = load_frag(lane_lo_b, lane_hi_b, kOffB, (H + t) * 16);
-    sa[t] = scale_of(swa, t, TM, a_upper);
-    sb[H + t] = scale_of(swb, H + t, TN, b_upper);
+    for (int t = 0; t < H; ++t) {
+      fa[t] = load_frag(lane_lo_a, lane_hi_a, 0, t * 16);
+      fb[H + t] = load_frag(lane_lo_b, lane_hi_b, kOffB, (H + t) * 16);
+#pragma unroll
+      for (int c = 0; c < KC; ++c) {
+        sa[c][t] = scale_bits(wa.w[c][t], c, 0);
+        sb[c][H + t] = scale_bits(wb.w[c][t], c, 0);
+      }
+    }
   }
 
   int slot = 0;  // ring slot of step ks
@@ -225,36 +260,59 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     const uint32_t cla = cur + lane_lo_a, cha = cur + lane_hi_a, clb = cur + lane_lo_b, chb = cur + lane_hi_b;
     const uint32_t nla = nxt + lane_lo_a, nha = nxt + lane_hi_a, nlb = nxt + lane_lo_b, nhb = nxt + lane_hi_b;
     int n_dma = 0;
+    HalfWords hw;  // scale words of the half a quadrant brings in
     __builtin_amdgcn_sched_barrier(0);
-    // H*H MFMAs over a tiles i0.., b tiles j0.. with the b tile as the outer index (the b half
-    // of a step's first quadrant is the one requested last); `after(q)` follows MFMA number q
+    // MFMAs over a tiles i0.., b tiles j0.. with the b tile as the outer index (the b half of a
+    // step's first quadrant is the one requested last); with FP4 first all tiles with the first
+    // 128 elements of the step, then all with the second, so that the two MFMAs into one
+    // accumulator are 16 apart.  `after(q)` follows the last MFMA of time slot q (one e4m3 MFMA
+    // or two e2m1 MFMAs, the same number of cycles).
     auto quadrant = [&](auto i0_tag, auto j0_tag, auto&& after) {
       constexpr int i0 = decltype(i0_tag)::value, j0 = decltype(j0_tag)::value;
 #pragma unroll
-      for (int q = 0; q < H * H; ++q) {
-        const int i = i0 + q % H, j = j0 + q / H;
+      for (int q = 0; q < H * H * KC; ++q) {
+        const int c = q / (H * H), t = q % (H * H);
+        const int i = i0 + t % H, j = j0 + t / H;
         // B fragment as the row operand: acc[i][j][v] = D[m = l16][n = 4*kq + v] of the tile
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], fa[i], acc[i][j], 0, 0, 0, sb[j], 0, sa[i]);
-        after(q);
+        if constexpr (!FP4) {
+          const v8i vb = __builtin_shufflevector(fb[j].lo, fb[j].hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          const v8i va = __builtin_shufflevector(fa[i].lo, fa[i].hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vb, va, acc[i][j], 0, 0, 0, sb[0][j], 0, sa[0][i]);
+        } else {
+          // Written as assembly with the accumulator tied in place: left to the register
+          // allocator, the two MFMAs per accumulator and step end up with different source
+          // and destination registers and copies through VGPRs (60 moves per step).
+          const v4i pb = c == 0 ? fb[j].lo : fb[j].hi, pa = c == 0 ? fa[i].lo : fa[i].hi;
+          asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+                       : "+a"(acc[i][j])
+                       : "v"(pb), "v"(pa), "v"(sb[c][j]), "v"(sa[c][i]));
+        }
+        if (q % KC == KC - 1) after(q / KC);
         __builtin_amdgcn_sched_barrier(0);
       }
     };
     auto dma = [&]() {
       if (n_dma < kLoadsPerStep) fetch_one(n_dma++, kn, cur);
     };
-    // ---- before the bar: (lo,hi) pulls b[lo], (lo,lo) pulls a[hi]
+    // ---- before the bar: (lo,hi) pulls b[lo], (lo,lo) pulls a[hi], both from this step's slot
     quadrant(kLo, kHi, [&](int q) {
-      if (q % H == 0) {
-        const int t = q / H;
-        fb[t] = load_frag(clb, chb, kOffB, t * 16);
-        sb[t] = scale_of(swb, t, TN, b_upper);
+      if (q == 0) hw = read_half_scales(cur + sc_lane_b, 0);
+      if (q % H == 0) fb[q / H] = load_frag(clb, chb, kOffB, (q / H) * 16);
+      if (q == H * H - 1) {
+#pragma unroll
+        for (int c = 0; c < KC; ++c)
+#pragma unroll
+          for (int t = 0; t < H; ++t) sb[c][t] = scale_bits(hw.w[c][t], c, ks);
       }
     });
     quadrant(kLo, kLo, [&](int q) {
-      if (q % (H - 1) == 0 && q / (H - 1) < H) {
-        const int t = H + q / (H - 1);
-        fa[t] = load_frag(cla, cha, 0, t * 16);
-        sa[t] = scale_of(swa, t, TM, a_upper);
+      if (q == 0) hw = read_half_scales(cur + sc_lane_a, 1);
+      if (q % (H - 1) == 0 && q / (H - 1) < H) fa[H + q / (H - 1)] = load_frag(cla, cha, 0, (H + q / (H - 1)) * 16);
+      if (q == H * H - 1) {
+#pragma unroll
+        for (int c = 0; c < KC; ++c)
+#pragma unroll
+          for (int t = 0; t < H; ++t) sa[c][H + t] = scale_bits(hw.w[c][t], c, ks);
       }
     });
     // every fragment of this step has been requested; once they are in, the slot is free
@@ -262,38 +320,39 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     // ---- behind the bar: (hi,hi) reloads a[lo], (hi,lo) reloads b[hi], both from step ks+1
-    constexpr int kFirstFrag = H > 2 ? 2 : 1, kFragEvery = H > 2 ? 3 : 1;
+    constexpr int kFirstFrag = H > 2 ? 1 : 0, kFragEvery = H > 2 ? 3 : 1;
     quadrant(kHi, kHi, [&](int q) {
-      if (q == 0) swb = read_scales(nxt + sc_lane_b);
-      if (q == (H > 2 ? 1 : 0)) swa = read_scales(nxt + sc_lane_a);
+      if (q == 0) hw = read_half_scales(nxt + sc_lane_a, 0);
       const int f = (q - kFirstFrag) / kFragEvery;
       if (q >= kFirstFrag && (q - kFirstFrag) % kFragEvery == 0 && f < H) fa[f] = load_frag(nla, nha, 0, f * 16);
-      else if (q >= 2 || H == 2) dma();
+      else if (q >= 1) dma();
       if (q == H * H - 1) {
 #pragma unroll
-        for (int t = 0; t < H; ++t) sa[t] = scale_of(swa, t, TM, a_upper);
+        for (int c = 0; c < KC; ++c)
+#pragma unroll
+          for (int t = 0; t < H; ++t) sa[c][t] = scale_bits(hw.w[c][t], c, ks + 1);
       }
     });
 #pragma unroll
     for (int t = 0; t < kLoadsPerStep / 2; ++t)
       if (n_dma < kLoadsPerStep / 2) dma();
     quadrant(kHi, kLo, [&](int q) {
-      if (q % H == 0) {
-        const int t = H + q / H;
-        fb[t] = load_frag(nlb, nhb, kOffB, t * 16);
-      } else {
-        dma();
-      }
+      if (q == 0) hw = read_half_scales(nxt + sc_lane_b, 1);
+      if (q % H == 0) fb[H + q / H] = load_frag(nlb, nhb, kOffB, (H + q / H) * 16);
+      else dma();
       if (q == H * H - 1) {
 #pragma unroll
-        for (int t = 0; t < H; ++t) sb[H + t] = scale_of(swb, H + t, TN, b_upper);
+        for (int c = 0; c < KC; ++c)
+#pragma unroll
+          for (int t = 0; t < H; ++t) sb[c][H + t] = scale_bits(hw.w[c][t], c, ks + 1);
       }
     });
 #pragma unroll
     for (int t = 0; t < kLoadsPerStep; ++t) dma();
   } while (++ks < k_steps);
   // the clamped refills of the last steps may still be landing: the epilogue reuses the LDS
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // (the no-ops cover the distance an assembly-written MFMA needs before its result is read)
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
   // ---- epilogue: fp32 -> bf16 (v_cvt_pk_bf16_f32, round to nearest even) and out through LDS.
@@ -333,17 +392,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4>
 int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N,
                 int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream) {
   const int tiles_m = (int)ceil_div(M, BM), tiles_n = (int)ceil_div(N, BN);
-  size_t lds_bytes = (size_t)NST * (((BM + BN) / kGroupRows) * kGroupStride + 2048);  // NST K-steps: panels + scale slots
+  // NST K-steps: panels + scale slots (1 KiB per operand and 128-element chunk of the step)
+  size_t lds_bytes = (size_t)NST * (((BM + BN) / kGroupRows) * kGroupStride + 2048 * (FP4 ? 2 : 1));
   const size_t epi_bytes = (size_t)WAVES_M * WAVES_N * (BM / WAVES_M) * ((BN / WAVES_N) * 2 + 16);  // epilogue staging
   if (lds_bytes < epi_bytes) lds_bytes = epi_bytes;
   // A grid that fits the chip once should land one workgroup per CU: asking for more than half
   // of the LDS keeps the dispatcher from pairing two workgroups on one CU while others idle.
   if ((int64_t)tiles_m * tiles_n <= device_facts().cu_count && lds_bytes < 82 * 1024) lds_bytes = 82 * 1024;
-  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST>;
+  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST, FP4>;
   if (lds_bytes > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess)
@@ -354,26 +414,42 @@ int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const ui
   return launch_status();
 }
 
+// Shared argument checks and tile choice.  K counts elements, lda/ldb bytes.
+template <bool FP4>
+int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N, int64_t K,
+            int64_t lda, int64_t ldb, void* out, int64_t ldo, dt_stream_t stream) {
+  if (M < 0 || N < 0 || K < 0) return DT_ERR_INVALID_SHAPE;
+  if (M == 0 || N == 0) return DT_OK;
+  if (K == 0 || K % 128 != 0) return DT_ERR_INVALID_SHAPE;  // one scaled MFMA covers 128 elements
+  const int64_t k_bytes = FP4 ? K / 2 : K;
+  if (N % 4 != 0 || ldo % 4 != 0 || ldo < N || lda < k_bytes || ldb < k_bytes) return DT_ERR_INVALID_SHAPE;
+  if (M > 0x7FFFFF00ll || N > 0x7FFFFF00ll || K > 0x7FFFFF00ll) return DT_ERR_INVALID_SHAPE;
+  if (!a || !b || !sfa || !sfb || !out) return DT_ERR_NULL_POINTER;
+  if (!aligned(a, 16) || !aligned(b, 16) || lda % 16 != 0 || ldb % 16 != 0) return DT_ERR_MISALIGNED;
+  if (!aligned(out, 8) || !aligned(sfa, 4) || !aligned(sfb, 4)) return DT_ERR_MISALIGNED;
+  // per-lane byte offsets into A and B are 32 bits wide
+  if ((M - 1) * lda + k_bytes > 0xFFFFFFFFll || (N - 1) * ldb + k_bytes > 0xFFFFFFFFll) return DT_ERR_INVALID_SHAPE;
+  const uint8_t* A = static_cast<const uint8_t*>(a);
+  const uint8_t* B = static_cast<const uint8_t*>(b);
+  hipStream_t s = as_hip(stream);
+  const int variant = tuning("gemm.variant");
+  const int64_t tiles256 = ceil_div(M, 256) * ceil_div(N, 256);
+  const bool big = variant == 2 || (variant == 0 && tiles256 >= device_facts().cu_count / 2);
+  // <tile M, tile N, waves M, waves N, LDS ring slots, e2m1 operands>
+  if (big) return launch_gemm<256, 256, 2, 2, 2, FP4>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  return launch_gemm<128, 128, 2, 2, 4, FP4>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+}
+
 }  // namespace dt
 
 extern "C" int dt_mx_fp8_bf16(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M,
                               int64_t N, int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo,
                               dt_stream_t stream) {
-  if (M < 0 || N < 0 || K < 0) return DT_ERR_INVALID_SHAPE;
-  if (M == 0 || N == 0) return DT_OK;
-  if (K == 0 || K % dt::kBK != 0) return DT_ERR_INVALID_SHAPE;
-  if (N % 4 != 0 || ldo % 4 != 0 || ldo < N || lda < K || ldb < K) return DT_ERR_INVALID_SHAPE;
-  if (M > 0x7FFFFF00ll || N > 0x7FFFFF00ll || K > 0x7FFFFF00ll) return DT_ERR_INVALID_SHAPE;
-  if (!a || !b || !sfa || !sfb || !out) return DT_ERR_NULL_POINTER;
-  if (!dt::aligned(a, 16) || !dt::aligned(b, 16) || lda % 16 != 0 || ldb % 16 != 0) return DT_ERR_MISALIGNED;
-  if (!dt::aligned(out, 8) || !dt::aligned(sfa, 4) || !dt::aligned(sfb, 4)) return DT_ERR_MISALIGNED;
-  const uint8_t* A = static_cast<const uint8_t*>(a);
-  const uint8_t* B = static_cast<const uint8_t*>(b);
-  hipStream_t s = dt::as_hip(stream);
-  const int variant = dt::tuning("gemm.variant");
-  const int64_t tiles256 = dt::ceil_div(M, 256) * dt::ceil_div(N, 256);
-  const bool big = variant == 2 || (variant == 0 && tiles256 >= dt::device_facts().cu_count / 2);
-  // <tile M, tile N, waves M, waves N, LDS ring slots>
-  if (big) return dt::launch_gemm<256, 256, 2, 2, 2>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
-  return dt::launch_gemm<128, 128, 2, 2, 4>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  return dt::mx_gemm<false>(a, b, sfa, sfb, M, N, K, lda, ldb, out, ldo, stream);
+}
+
+extern "C" int dt_mx_fp4_bf16(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M,
+                              int64_t N, int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo,
+                              dt_stream_t stream) {
+  return dt::mx_gemm<true>(a, b, sfa, sfb, M, N, K, lda, ldb, out, ldo, stream);
 }

@@ -290,8 +290,50 @@ Tensor mx_fp8_bf16(Tensor a, Tensor b, Tensor a_scale, Tensor b_scale) {
   return out;
 }
 
+// ------------------------------------------------------------------------ mx_fp4_bf16
+// src/mx_fp8_bf16.cu:243-271.  a [M, K/2] and b [K/2, N] with stride(0) == 1 hold two e2m1
+// values per byte, the even element in the low nibble (uint8 or float4_e2m1fn_x2 storage);
+// K = 2 * a.size(1) as at :254.  The reference runs no operand checks here; these are the
+// checks of mx_fp8_bf16 (:168-214) applied to the unpacked K.
+Tensor mx_fp4_bf16(Tensor a, Tensor b, Tensor a_scale, Tensor b_scale) {
+  TORCH_CHECK(a.is_cuda(), "a must be CUDA tensor");
+  TORCH_CHECK(b.is_cuda(), "b must be CUDA tensor");
+  TORCH_CHECK(a_scale.is_cuda(), "a_scale must be CUDA tensor");
+  TORCH_CHECK(b_scale.is_cuda(), "b_scale must be CUDA tensor");
+  TORCH_CHECK(a.dim() == 2, "a must be a matrix");
+  TORCH_CHECK(b.dim() == 2, "b must be a matrix");
+  auto packed = [](const Tensor& t) {
+    return t.scalar_type() == at::kByte || t.scalar_type() == at::ScalarType::Float4_e2m1fn_x2;
+  };
+  TORCH_CHECK(packed(a) && packed(b), "a and b must hold packed e2m1 pairs (uint8 or float4_e2m1fn_x2)");
+  TORCH_CHECK(a_scale.element_size() == 1 && b_scale.element_size() == 1, "scales must be E8M0 bytes");
+  const int64_t M = a.size(0), Kp = a.size(1), K = 2 * Kp, N = b.size(1);
+  TORCH_CHECK(b.size(0) == Kp, "Incompatible matrix dimensions: a is ", M, "x", Kp, " but b is ", b.size(0), "x", N);
+  TORCH_CHECK(N % 8 == 0, "N must be a multiple of 16 but got, ", N);
+  TORCH_CHECK(K % 128 == 0, "K must be a multiple of 128 but got ", K);
+  TORCH_CHECK(reinterpret_cast<std::uintptr_t>(a.data_ptr()) % 16 == 0, "Input tensor 'a' must be 16-byte aligned");
+  TORCH_CHECK(reinterpret_cast<std::uintptr_t>(b.data_ptr()) % 16 == 0, "Input tensor 'b' must be 16-byte aligned");
+  auto ceil_div = [](int64_t x, int64_t y) { return (x + y - 1) / y; };
+  const int64_t num_k_blocks = ceil_div(K, 32);
+  const int64_t expected_a = 128 * ceil_div(M, 128) * num_k_blocks;
+  TORCH_CHECK(a_scale.numel() == expected_a, "Expected a_scale_size to be ", expected_a, " but got ", a_scale.numel());
+  const int64_t expected_b = 128 * ceil_div(N, 128) * num_k_blocks;
+  TORCH_CHECK(b_scale.numel() == expected_b, "Expected b_scale_size to be ", expected_b, " but got ", b_scale.numel());
+  TORCH_CHECK(a.stride(1) == 1, "Input tensor 'a' must be contiguous in the K dimension (row-major)");
+  TORCH_CHECK(b.stride(0) == 1, "Input tensor 'b' must be contiguous in the K dimension (column-major)");
+  TORCH_CHECK(a_scale.is_contiguous() && b_scale.is_contiguous(), "scales must be contiguous");
+  Ctx ctx(a);
+  Tensor out = at::empty({M, N}, a.options().dtype(at::kBFloat16));
+  if (M == 0 || N == 0) return out;
+  const int64_t lda = M > 1 ? a.stride(0) : Kp, ldb = N > 1 ? b.stride(1) : Kp;
+  check_status(dt_mx_fp4_bf16(a.data_ptr(), b.data_ptr(), static_cast<const uint8_t*>(a_scale.data_ptr()),
+                              static_cast<const uint8_t*>(b_scale.data_ptr()), M, N, K, lda, ldb, out.data_ptr(), N,
+                              ctx.stream),
+               "mx_fp4_bf16");
+  return out;
+}
+
 // ----------------------------------------------------------- schemas kept, not built
-Tensor mx_fp4_bf16(Tensor, Tensor, Tensor, Tensor) { TORCH_CHECK(false, "Not built for this platform!"); }
 Tensor keyed_random_uniform(Tensor, int64_t) { TORCH_CHECK(false, "Not built for this platform!"); }
 Tensor sweep_mm(Tensor, Tensor, Tensor, Tensor, std::optional<Tensor>, at::ScalarType, bool, int64_t, int64_t, int64_t,
                 bool, int64_t) {

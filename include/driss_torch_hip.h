@@ -167,6 +167,16 @@ DT_API int dt_mx_fp8_bf16(const void* a, const void* b, const uint8_t* sfa, cons
                           int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, void* out,
                           int64_t ldo, dt_stream_t stream);
 
+/* ------------------------------------------------------------------ mx_fp4_bf16 ------
+ * The same product with e2m1 operands.  Replaces driss_torch::mx_fp4_bf16,
+ * src/mx_fp8_bf16.cu:243-271.  a: [M, K/2] bytes, b: [N, K/2] bytes (the reference's
+ * [K/2, N] tensor with stride(0)==1), two e2m1 values per byte with the even element in
+ * the low nibble; K counts elements, lda / ldb bytes.  Scales, alignment and shape
+ * rules as for dt_mx_fp8_bf16 (K % 128 == 0).                                           */
+DT_API int dt_mx_fp4_bf16(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb,
+                          int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, void* out,
+                          int64_t ldo, dt_stream_t stream);
+
 /* ---------------------------------------------------------------- tuning -------------
  * Launch-shape knobs for benchmarking sweeps ("amax.blocks_per_cu", ...).  Returns DT_OK
  * or DT_ERR_INVALID_MODE for an unknown key.  Not part of the reference's surface.        */

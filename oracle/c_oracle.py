@@ -63,6 +63,12 @@ def lib() -> C.CDLL:
         L.dto_mx_gemm_ref.restype = None
         L.dto_mx_gemm_ref.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]
         L.dto_mx_dequant.restype, L.dto_mx_dequant.argtypes = None, [vp, vp, i64, i64, i32, vp]
+        L.dto_e2m1_to_f32.restype, L.dto_e2m1_to_f32.argtypes = C.c_float, [C.c_uint8]
+        L.dto_f32_to_e2m1.restype, L.dto_f32_to_e2m1.argtypes = C.c_uint8, [C.c_float]
+        L.dto_fp4_unpack.restype, L.dto_fp4_unpack.argtypes = None, [vp, i64, i64, vp]
+        L.dto_mx_fp4_quantize.restype, L.dto_mx_fp4_quantize.argtypes = None, [vp, i64, i64, vp, vp]
+        L.dto_mx_fp4_gemm_ref.restype = None
+        L.dto_mx_fp4_gemm_ref.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]
         _lib = L
     return _lib
 
@@ -157,4 +163,41 @@ def mx_dequant(data: torch.Tensor, scale: torch.Tensor, out_dtype: torch.dtype =
     R, Cc = data.shape
     out = torch.empty((R, Cc), dtype=torch.float32)
     lib().dto_mx_dequant(_p(data), _p(scale), R, Cc, _OUT_DTYPE[out_dtype], _p(out))
+    return out
+
+
+def e2m1_to_f32(code: int) -> float:
+    return lib().dto_e2m1_to_f32(code)
+
+
+def f32_to_e2m1(x: float) -> int:
+    return lib().dto_f32_to_e2m1(x)
+
+
+def fp4_unpack(packed: torch.Tensor) -> torch.Tensor:
+    """[R, C/2] uint8 (even element in the low nibble) -> fp32 [R, C]"""
+    packed = _cpu(packed)
+    R, Ch = packed.shape
+    out = torch.empty((R, 2 * Ch), dtype=torch.float32)
+    lib().dto_fp4_unpack(_p(packed), R, 2 * Ch, _p(out))
+    return out
+
+
+def mx_fp4_quantize(x: torch.Tensor):
+    """Test-operand generator: fp32 [R, C] -> (packed e2m1 [R, C/2] uint8, E8M0 [R, C/32] uint8)."""
+    x = _cpu(x.float())
+    R, Cc = x.shape
+    data = torch.empty((R, Cc // 2), dtype=torch.uint8)
+    scale = torch.empty((R, Cc // 32), dtype=torch.uint8)
+    lib().dto_mx_fp4_quantize(_p(x), R, Cc, _p(data), _p(scale))
+    return data, scale
+
+
+def mx_fp4_gemm_ref(a: torch.Tensor, bt: torch.Tensor, sfa_blocked: torch.Tensor, sfb_blocked: torch.Tensor) -> torch.Tensor:
+    """a [M,K/2], bt [N,K/2] packed e2m1, blocked scales -> fp32 [M,N] (float64 accumulation)."""
+    a, bt = _cpu(a), _cpu(bt)
+    M, Kp = a.shape
+    N = bt.shape[0]
+    out = torch.empty((M, N), dtype=torch.float32)
+    lib().dto_mx_fp4_gemm_ref(_p(a), _p(bt), _p(_cpu(sfa_blocked)), _p(_cpu(sfb_blocked)), M, N, 2 * Kp, Kp, Kp, _p(out))
     return out

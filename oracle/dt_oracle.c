@@ -19,12 +19,19 @@
  *   blocked scale layout     test/test_mx.py:28-32 (transformer_nuggets to_blocked, absent from the
  *                            reference tree, unpinned), length check src/mx_fp8_bf16.cu:197-205
  *   MX GEMM                  test/test_mx.py:34-39, src/mx_fp8_bf16.cu:217-241
+ *   MXFP4 GEMM               test/test_mx.py:17-39 (format "fp4"), src/mx_fp8_bf16.cu:243-271; e2m1 per the
+ *                            OCP Microscaling Formats v1.0 element table; two values per byte with the
+ *                            even element in the low nibble (the packing of torchao's MXTensor data that
+ *                            the reference's test hands to the kernel; torchao absent, unpinned version)
  *
  * Pinning (see tests/): fp8/bf16 converts are checked exhaustively against torch's CPU
  * `.to(float8_*)` over all 2^16 bf16 patterns and a dense fp32 sweep, and against the
  * known-answer vectors in tests/golden/; amax/scale/cast against the eager formulation;
  * the MX exponent against ceil(log2) in exact (float64 / integer) arithmetic; to_blocked
  * against the view/permute formulation; the GEMM against brute force and float64 matmul.
+ * The e2m1 decode is pinned by the eight magnitudes of the OCP table and the sign bit; the fp4
+ * quantizer below only manufactures test operands (floor-exponent scaling as in the OCP
+ * specification) and is "parity unpinned" against torchao's to_mx, which no op of the path calls.
  * Documented choices where the third-party oracle (torchao) is version dependent and no
  * vector in the reference pins it ("parity unpinned" corners): a block holding a NaN gets
  * scale byte 255 and an all-NaN payload; scale byte 0 decodes to 2^-127 (its E8M0 value);
@@ -398,5 +405,82 @@ DTO_EXPORT void dto_mx_dequant(const uint8_t* data, const uint8_t* scale, int64_
       float v = out_dtype == DTO_E5M2 ? dto_e5m2_to_f32(b) : dto_e4m3fn_to_f32(b);
       uint8_t s = scale[r * nb + c / 32];
       out[r * C + c] = s == 255 ? u2f(0x7FC00000u) : (float)ldexp((double)v, (int)s - 127);
+    }
+}
+
+/* ------------------------------------------------------------------ MXFP4 (e2m1) ------ */
+/* e2m1: sign, 2 exponent bits (bias 1), 1 mantissa bit; no infinities, no NaNs. */
+DTO_EXPORT float dto_e2m1_to_f32(uint8_t code) {
+  int e = (code >> 1) & 3, m = code & 1;
+  float v = e == 0 ? 0.5f * (float)m : ldexpf(1.0f + 0.5f * (float)m, e - 1);
+  return (code & 8) ? -v : v;
+}
+
+/* round to nearest even onto the e2m1 grid {0, .5, 1, 1.5, 2, 3, 4, 6}, saturating */
+DTO_EXPORT uint8_t dto_f32_to_e2m1(float f) {
+  uint8_t s = (f2u(f) >> 31) ? 8 : 0;
+  float a = fabsf(f);
+  if (!(a == a)) return (uint8_t)(s | 7);
+  static const float grid[8] = {0.f, 0.5f, 1.f, 1.5f, 2.f, 3.f, 4.f, 6.f};
+  int best = 7;
+  for (int i = 0; i < 7; ++i) {
+    float mid = 0.5f * (grid[i] + grid[i + 1]);
+    if (a < mid || (a == mid && (i & 1) == 0)) { best = i; break; }
+  }
+  return (uint8_t)(s | best);
+}
+
+/* packed [R, C/2] -> fp32 [R, C] (element 2j in the low nibble of byte j) */
+DTO_EXPORT void dto_fp4_unpack(const uint8_t* packed, int64_t R, int64_t C, float* out) {
+  for (int64_t r = 0; r < R; ++r)
+    for (int64_t c = 0; c < C; ++c) {
+      uint8_t b = packed[r * (C / 2) + c / 2];
+      out[r * C + c] = dto_e2m1_to_f32((c & 1) ? (uint8_t)(b >> 4) : (uint8_t)(b & 15));
+    }
+}
+
+/* Test-operand generator: fp32 [R, C] -> packed e2m1 [R, C/2] + E8M0 [R, C/32], shared
+ * exponent floor(log2(blockmax)) - 2 (2 = emax of e2m1), zero blocks get byte 0. */
+DTO_EXPORT void dto_mx_fp4_quantize(const float* x, int64_t R, int64_t C, uint8_t* data, uint8_t* scale) {
+  for (int64_t r = 0; r < R; ++r)
+    for (int64_t kb = 0; kb < C / 32; ++kb) {
+      const float* p = x + r * C + kb * 32;
+      float m = 0.f;
+      for (int i = 0; i < 32; ++i) m = fmaxf(m, fabsf(p[i]));
+      int e = -127;
+      if (m > 0.f) { int ex; frexpf(m, &ex); e = ex - 1 - 2; }
+      if (e < -127) e = -127;
+      if (e > 127) e = 127;
+      scale[r * (C / 32) + kb] = (uint8_t)(e + 127);
+      for (int i = 0; i < 32; i += 2) {
+        uint8_t lo = dto_f32_to_e2m1(ldexpf(p[i], -e)), hi = dto_f32_to_e2m1(ldexpf(p[i + 1], -e));
+        data[r * (C / 2) + kb * 16 + i / 2] = (uint8_t)(lo | (hi << 4));
+      }
+    }
+}
+
+/* out[M,N] = sum_k a[m,k] 2^(sfa-127) * b[n,k] 2^(sfb-127): a [M, K/2], bt [N, K/2] packed
+ * e2m1 (row strides lda, ldb bytes), scales in the blocked layout; float64 accumulation. */
+DTO_EXPORT void dto_mx_fp4_gemm_ref(const uint8_t* a, const uint8_t* bt, const uint8_t* sfa,
+                                    const uint8_t* sfb, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                    int64_t ldb, float* out) {
+  int64_t KB = K / 32;
+  float lut[16];
+  for (int i = 0; i < 16; ++i) lut[i] = dto_e2m1_to_f32((uint8_t)i);
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m)
+    for (int64_t n = 0; n < N; ++n) {
+      double acc = 0.0;
+      for (int64_t kb = 0; kb < KB; ++kb) {
+        double part = 0.0;
+        for (int64_t j = kb * 16; j < kb * 16 + 16; ++j) {
+          uint8_t x = a[m * lda + j], y = bt[n * ldb + j];
+          part += (double)lut[x & 15] * (double)lut[y & 15] + (double)lut[x >> 4] * (double)lut[y >> 4];
+        }
+        int ea = (int)sfa[dto_blocked_offset(m, kb, KB)] - 127;
+        int eb = (int)sfb[dto_blocked_offset(n, kb, KB)] - 127;
+        acc += ldexp(part, ea + eb);
+      }
+      out[m * N + n] = (float)acc;
     }
 }

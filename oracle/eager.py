@@ -150,3 +150,24 @@ def compute_error(ref: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """torchao compute_error (test/test_mx.py:6,39): SQNR in dB."""
     ref, out = ref.to(torch.float64), out.to(torch.float64)
     return 20 * torch.log10(torch.linalg.norm(ref) / torch.linalg.norm(ref - out))
+
+
+# ------------------------------------------------------------------------- MXFP4 (e2m1)
+# OCP Microscaling Formats v1.0, FP4 E2M1 element table: code -> value
+E2M1_VALUES = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+
+
+def fp4_unpack(packed_u8: torch.Tensor) -> torch.Tensor:
+    """[R, C/2] uint8 -> fp32 [R, C]; element 2j is the low nibble of byte j (the packing of the
+    MXTensor data the reference's test passes to mx_fp4_bf16, test/test_mx.py:23-26)."""
+    lut = torch.tensor(E2M1_VALUES + [-v for v in E2M1_VALUES], dtype=torch.float32)
+    lo = lut[(packed_u8 & 15).long()]
+    hi = lut[(packed_u8 >> 4).long()]
+    return torch.stack([lo, hi], dim=-1).reshape(packed_u8.shape[0], -1)
+
+
+def mx_fp4_dequant(packed_u8: torch.Tensor, scale_u8: torch.Tensor, block: int = 32) -> torch.Tensor:
+    v = fp4_unpack(packed_u8)
+    R, Cc = v.shape
+    s = torch.exp2(scale_u8.view(R, Cc // block, 1).double() - 127.0)
+    return (v.view(R, Cc // block, block).double() * s).view(R, Cc)

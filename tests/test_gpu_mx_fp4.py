@@ -1,0 +1,164 @@
+"""GPU parity of mx_fp4_bf16 (e2m1 operands, E8M0 block-32 scales) against the CPU oracle, on the
+reference's size list (test/test_mx.py:42-59 with format "fp4").  Operands come from the oracle's
+fp4 generator: the reference takes them from torchao's MXTensor, and no op of the path makes them."""
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from oracle import eager
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def d(gpu_device):
+    import driss_torch_amd
+
+    return driss_torch_amd
+
+
+@pytest.fixture(scope="module")
+def cabi(gpu_device):
+    from driss_torch_amd import cabi as c
+
+    return c
+
+
+def _operands(M, K, N, seed, dist="rand"):
+    mk = util.uniform if dist == "rand" else util.normal
+    a, sa = co.mx_fp4_quantize(mk((M, K), seed, torch.float32))
+    b, sb = co.mx_fp4_quantize(mk((N, K), seed + 1, torch.float32) * 3)
+    return a, sa, b, sb
+
+
+def _run(d, a, sa, b, sb):
+    return d.mx_fp4_bf16(a.cuda(), b.cuda().t(), d.to_blocked(sa.cuda()), d.to_blocked(sb.cuda()))
+
+
+def _check(d, M, K, N, seed, dist):
+    a, sa, b, sb = _operands(M, K, N, seed, dist)
+    out = _run(d, a, sa, b, sb)
+    assert out.shape == (M, N) and out.dtype == torch.bfloat16
+    da, db = eager.mx_fp4_dequant(a, sa), eager.mx_fp4_dequant(b, sb)
+    ref = da @ db.T
+    got = out.cpu().double()
+    # Tolerance as for the e4m3 GEMM: products of e2m1 values are exact in fp32, the accumulation
+    # is fp32 and the store rounds to bf16 (relative 2^-9), so every entry lies within
+    # 2^-8 * sum_k |a||b| of the exact product; SQNR against the exact product > 50 dB (the
+    # reference asks 80 dB against a bf16 matmul of the same operands, test/test_mx.py:64).
+    bound = da.abs() @ db.abs().T
+    err = (got - ref).abs()
+    assert (err <= bound * 2**-8 + 1e-30).all(), f"max rel {(err / bound).max().item():.3e}"
+    assert eager.compute_error(ref, got).item() > 50
+    return out
+
+
+@pytest.mark.parametrize("size", [(128, 128, 128), (256, 256, 256), (384, 384, 384), (512, 512, 512), (768, 768, 768),
+                                  (1024, 1024, 1024), (128, 256, 384), (256, 384, 512), (129, 256, 384), (133, 512, 528)],
+                         ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+@pytest.mark.parametrize("dist", ["rand", "randn"])
+def test_mx_fp4_gemm_reference_sizes(d, size, dist):
+    M, K, N = size
+    _check(d, M, K, N, 900 + M + N, dist)
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("size", [(128, 128, 128), (512, 256, 640), (133, 640, 528), (300, 1152, 264), (64, 2048, 8)])
+def test_mx_fp4_gemm_both_tile_shapes(d, cabi, variant, size):
+    """K = 128, 640, 1152 end in a half-filled 256-element step; K = 256, 2048 do not"""
+    cabi.set_tuning("gemm.variant", variant)
+    try:
+        _check(d, *size, 950, "randn")
+    finally:
+        cabi.set_tuning("gemm.variant", 0)
+
+
+def test_mx_fp4_gemm_bit_exact_when_sums_fit_fp32(d):
+    """sparse operands and a narrow scale range: every product and every partial sum is a multiple
+    of 2^-6 below 2^12, exact in fp32 in any order, so the result must equal the C oracle's float64
+    reference rounded once to bf16, bit for bit, for full and half-filled last steps"""
+    g = util.gen(91)
+    for (M, K, N) in ((160, 384, 136), (130, 512, 264)):
+        a = torch.randint(0, 16, (M, K), generator=g, dtype=torch.uint8) * (torch.rand(M, K, generator=g) < 0.03)
+        b = torch.randint(0, 16, (N, K), generator=g, dtype=torch.uint8) * (torch.rand(N, K, generator=g) < 0.5)
+        ap = (a[:, 0::2] | (a[:, 1::2] << 4)).to(torch.uint8)
+        bp = (b[:, 0::2] | (b[:, 1::2] << 4)).to(torch.uint8)
+        sa = torch.randint(125, 130, (M, K // 32), generator=g, dtype=torch.uint8)
+        sb = torch.randint(125, 130, (N, K // 32), generator=g, dtype=torch.uint8)
+        out = _run(d, ap, sa, bp, sb)
+        ref = co.mx_fp4_gemm_ref(ap, bp, co.to_blocked(sa), co.to_blocked(sb))
+        assert torch.equal(out.cpu(), ref.bfloat16())
+
+
+def test_mx_fp4_gemm_scales_per_row_and_kblock(d):
+    M, K, N = 256, 640, 256
+    a, sa, b, sb = _operands(M, K, N, 93, "randn")
+    base = _run(d, a, sa, b, sb).float()
+    sa2 = sa.clone()
+    sa2[77, :] += 3
+    out = _run(d, a, sa2, b, sb).float()
+    assert torch.equal(out[77], base[77] * 8)
+    assert torch.equal(out[:77], base[:77]) and torch.equal(out[78:], base[78:])
+    for kb in (2, 5, 17, 19):  # K-blocks in the first and second half of a step, and in the half-filled last step
+        b2 = torch.zeros_like(b)
+        b2[:, kb * 16:(kb + 1) * 16] = b[:, kb * 16:(kb + 1) * 16]
+        out = _run(d, a, sa, b2, sb).cpu().double()
+        da = eager.mx_fp4_dequant(a, sa)[:, kb * 32:(kb + 1) * 32]
+        db = eager.mx_fp4_dequant(b, sb)[:, kb * 32:(kb + 1) * 32]
+        ref, bound = da @ db.T, da.abs() @ db.abs().T
+        assert ((out - ref).abs() <= bound * 2**-8).all()
+
+
+def test_mx_fp4_gemm_strided_a_and_float4_storage(d):
+    M, K, N = 192, 512, 136
+    a, sa, b, sb = _operands(M, K, N, 95, "randn")
+    wide = torch.zeros((M, K // 2 + 64), dtype=torch.uint8, device="cuda")
+    wide[:, :K // 2] = a.cuda()
+    av = wide[:, :K // 2]  # row stride K/2 + 64 bytes
+    want = _run(d, a, sa, b, sb)
+    got = d.mx_fp4_bf16(av, b.cuda().t(), d.to_blocked(sa.cuda()), d.to_blocked(sb.cuda()))
+    assert torch.equal(got, want)
+    if hasattr(torch, "float4_e2m1fn_x2"):
+        got = d.mx_fp4_bf16(a.cuda().view(torch.float4_e2m1fn_x2), b.cuda().view(torch.float4_e2m1fn_x2).t(),
+                            d.to_blocked(sa.cuda()), d.to_blocked(sb.cuda()))
+        assert torch.equal(got, want)
+
+
+def test_mx_fp4_gemm_argument_errors(d):
+    a, sa, b, sb = _operands(128, 256, 128, 97)
+    A, B, SA, SB = a.cuda(), b.cuda(), d.to_blocked(sa.cuda()), d.to_blocked(sb.cuda())
+    with pytest.raises(RuntimeError):
+        d.mx_fp4_bf16(A, B, SA, SB)  # b not K-contiguous
+    with pytest.raises(RuntimeError):
+        d.mx_fp4_bf16(A, B.t(), SA[:-1], SB)  # scale length for K = 2 * a.size(1)
+    with pytest.raises(RuntimeError):
+        d.mx_fp4_bf16(A[:, :96], B[:, :96].t(), SA, SB)  # K = 192 is not a multiple of 128
+    with pytest.raises(RuntimeError):
+        d.mx_fp4_bf16(A.view(torch.float8_e4m3fn), B.t(), SA, SB)
+
+
+def test_mx_fp4_gemm_compile(d):
+    a, sa, b, sb = _operands(256, 512, 384, 98)
+    args = (a.cuda(), b.cuda().t(), d.to_blocked(sa.cuda()), d.to_blocked(sb.cuda()))
+    torch._dynamo.reset()
+    fn = torch.compile(d.mx_fp4_bf16, fullgraph=True, backend="aot_eager")
+    assert torch.equal(fn(*args), d.mx_fp4_bf16(*args))
+
+
+def test_mx_fp4_gemm_full_size(d):
+    """8192^3; checked on sampled rows against the float64 dequantized product"""
+    M = N = K = 8192
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a = torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8, device="cuda")
+    b = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8, device="cuda")
+    sa = torch.randint(120, 134, (M, K // 32), generator=g, dtype=torch.uint8, device="cuda")
+    sb = torch.randint(120, 134, (N, K // 32), generator=g, dtype=torch.uint8, device="cuda")
+    out = d.mx_fp4_bf16(a, b.t(), d.to_blocked(sa), d.to_blocked(sb))
+    rows = torch.tensor([0, 1, 127, 128, 255, 256, 4095, 4096, 8000, 8191])
+    da = eager.mx_fp4_dequant(a[rows.cuda()].cpu(), sa[rows.cuda()].cpu())
+    cols = torch.arange(0, N, 61)
+    db = eager.mx_fp4_dequant(b[cols.cuda()].cpu(), sb[cols.cuda()].cpu())
+    ref, bound = da @ db.T, da.abs() @ db.abs().T
+    got = out[rows.cuda()][:, cols.cuda()].cpu().double()
+    assert ((got - ref).abs() <= bound * 2**-8).all()

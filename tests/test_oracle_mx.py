@@ -12,6 +12,7 @@ import torch
 
 from oracle import c_oracle as co
 from oracle import eager
+from tests import util
 
 GOLD = Path(__file__).parent / "golden"
 
@@ -146,3 +147,81 @@ def test_mx_gemm_scale_linearity():
     out = co.mx_gemm_ref(ad, bd, co.to_blocked(asc2), co.to_blocked(bsc))
     torch.testing.assert_close(out[7], base[7] * 2)
     assert torch.equal(out[:7], base[:7]) and torch.equal(out[8:], base[8:])
+
+
+# ----------------------------------------------------------------------------- MXFP4 (e2m1)
+def test_e2m1_decode_matches_the_ocp_table_and_closed_form():
+    """OCP Microscaling Formats v1.0, FP4 E2M1: magnitudes 0, .5, 1, 1.5, 2, 3, 4, 6; bit 3 is the sign"""
+    table = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+    for code in range(16):
+        s, e, m = code >> 3, (code >> 1) & 3, code & 1
+        closed = (m * 0.5) if e == 0 else (1 + m / 2) * 2.0 ** (e - 1)
+        closed = -closed if s else closed
+        got = co.e2m1_to_f32(code)
+        assert got == closed == (-table[code & 7] if s else table[code & 7])
+        assert math.copysign(1.0, got) == (-1.0 if s else 1.0)
+    assert eager.E2M1_VALUES == table
+
+
+def test_e2m1_encode_is_nearest_even_and_saturates():
+    grid = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+    g = util.gen(31)
+    xs = (torch.rand(4000, generator=g) * 8 - 1).tolist() + [0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0, 7.0, 1e9]
+    for x in xs:
+        for sign in (1.0, -1.0):
+            code = co.f32_to_e2m1(sign * x)
+            a = abs(x)
+            d = [abs(a - v) for v in grid]
+            best = min(d)
+            cands = [i for i, v in enumerate(d) if v == best]
+            want = cands[0] if len(cands) == 1 else [i for i in cands if i % 2 == 0][0]
+            assert code & 7 == want, (x, code)
+            assert (code >> 3) == (1 if math.copysign(1.0, sign * x) < 0 else 0)
+    for code in range(16):  # every code is a fixed point
+        assert co.f32_to_e2m1(co.e2m1_to_f32(code)) == code
+
+
+def test_fp4_unpack_low_nibble_first_c_vs_eager():
+    g = util.gen(32)
+    packed = torch.randint(0, 256, (37, 48), generator=g, dtype=torch.uint8)
+    a, b = co.fp4_unpack(packed), eager.fp4_unpack(packed)
+    assert torch.equal(a, b)
+    assert a[3, 10] == co.e2m1_to_f32(int(packed[3, 5]) & 15) and a[3, 11] == co.e2m1_to_f32(int(packed[3, 5]) >> 4)
+
+
+def test_fp4_operand_generator_properties():
+    x = util.normal((64, 256), 33, torch.float32)
+    x[5, 32:64] = 0.0
+    data, scale = co.mx_fp4_quantize(x)
+    assert data.shape == (64, 128) and scale.shape == (64, 8)
+    deq = eager.mx_fp4_dequant(data, scale).float()
+    blk = x.view(64, 8, 32)
+    amax = blk.abs().amax(-1)
+    # shared exponent floor(log2(amax)) - 2: the block maximum lands in [4, 8) before rounding
+    e = scale.double() - 127
+    nz = amax > 0
+    scaled_max = amax.double() / torch.exp2(e)
+    assert ((scaled_max[nz] >= 4) & (scaled_max[nz] < 8)).all()
+    assert (scale[5, 1] == 0) and (deq[5, 32:64] == 0).all()
+    # error: half a grid step (the widest is 2, between 4 and 6) of the block scale, saturation at 6
+    err = (deq.view(64, 8, 32) - blk).abs().double()
+    assert (err <= torch.exp2(e).unsqueeze(-1) * 2.0 + 1e-30).all()
+    # idempotent on its own output
+    d2, s2 = co.mx_fp4_quantize(deq)
+    assert torch.equal(eager.mx_fp4_dequant(d2, s2).float(), deq)
+
+
+def test_fp4_gemm_ref_against_float64_matmul_and_brute_force():
+    M, N, K = 70, 52, 384
+    a, sa = co.mx_fp4_quantize(util.normal((M, K), 34, torch.float32))
+    b, sb = co.mx_fp4_quantize(util.normal((N, K), 35, torch.float32) * 7)
+    ref = co.mx_fp4_gemm_ref(a, b, co.to_blocked(sa), co.to_blocked(sb))
+    want = eager.mx_fp4_dequant(a, sa) @ eager.mx_fp4_dequant(b, sb).T
+    assert torch.equal(ref, want.float())
+    m, n = 13, 41
+    acc = 0.0
+    for k in range(K):
+        av = co.e2m1_to_f32((int(a[m, k // 2]) >> (4 * (k & 1))) & 15) * 2.0 ** (int(sa[m, k // 32]) - 127)
+        bv = co.e2m1_to_f32((int(b[n, k // 2]) >> (4 * (k & 1))) & 15) * 2.0 ** (int(sb[n, k // 32]) - 127)
+        acc += av * bv
+    assert abs(ref[m, n].item() - acc) <= 1e-6 * abs(acc)
