@@ -26,6 +26,7 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 FP8_PEAK_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
+FP4_PEAK_TFLOPS = 10100.0   # MI355X dense fp4 MFMA
 MALL_BYTES = 256 << 20
 # HBM-side bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, each
 # scaled by what the same counter reads for a plain 128 MiB device copy (fetch x1.9996, write
@@ -257,6 +258,18 @@ def extra_kernels(torch, cabi, util, dev, K, W):
     rows.append({"kernel": "mx_fp8_bf16", "workload": "config 5: 8192^3 e4m3 x e4m3, E8M0 block-32 scales -> bf16",
                  "bound": "mfma", "avg_us": round(us, 2), "achieved_TFLOPs": round(tf, 1),
                  "frac_of_fp8_peak": round(tf / FP8_PEAK_TFLOPS, 4), "flops": flops})
+    # MXFP4 GEMM, same shape: random e2m1 codes and scale bytes (no op of the path produces fp4)
+    del a_data, b_data
+    g = torch.Generator(device=dev).manual_seed(5)
+    a4 = torch.randint(0, 256, (M, Kd // 2), generator=g, dtype=torch.uint8, device=dev)
+    b4 = torch.randint(0, 256, (N, Kd // 2), generator=g, dtype=torch.uint8, device=dev)
+    s4a = torch.randint(120, 134, (sfa.numel(),), generator=g, dtype=torch.uint8, device=dev)
+    s4b = torch.randint(120, 134, (sfb.numel(),), generator=g, dtype=torch.uint8, device=dev)
+    us = time_launches(lambda i: cabi.mx_fp4_bf16(a4, b4, s4a, s4b, out), 1, max(20, K // 2), max(30, W))
+    tf = flops / (us * 1e-6) / 1e12
+    rows.append({"kernel": "mx_fp4_bf16", "workload": "8192^3 e2m1 x e2m1, E8M0 block-32 scales -> bf16",
+                 "bound": "mfma", "avg_us": round(us, 2), "achieved_TFLOPs": round(tf, 1),
+                 "frac_of_fp4_peak": round(tf / FP4_PEAK_TFLOPS, 4), "flops": flops})
     return rows
 
 
