@@ -43,7 +43,7 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 // elements = two MFMAs: bytes 16g.. of the first half feed the first, bytes 64+16g.. the second,
 // which are the same two 16-byte reads a lane makes for e4m3.  Everything else (panels, DMA,
 // swizzle, ring, quadrant schedule, epilogue) is shared; a K-step carries twice the scales.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4, bool TOUCH>
 __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const uint8_t* __restrict__ sfa,
     const uint8_t* __restrict__ sfb, int M, int N, int K, int64_t lda, int64_t ldb, uint16_t* __restrict__ out,
@@ -148,6 +148,40 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
 #pragma unroll
     for (int n = 0; n < kLoadsPerStep; ++n) fetch_one(n, ks, buf);
   };
+  // L2 prefetch (TOUCH).  The refill of a stage is issued one K-step before it is needed, which
+  // is shorter than an L2 miss; and every panel line is an L2 miss for the first workgroup of
+  // the XCD that asks for it.  So each workgroup also "touches" lines of a K-step further ahead
+  // with one 4-byte LDS-DMA load per wave (no register destination; the bytes land in a dump
+  // area nobody reads).  The 4 tile columns that share an A panel inside an XCD (and the 8 tile
+  // rows that share a B panel) split the panel's lines between them: 64 lines of A and 32 of B
+  // per workgroup and step, 24 per wave.  A line nobody touched is merely slower.
+  constexpr int kTouch = TOUCH ? 1 : 0;       // touch loads per wave and step
+  constexpr int kTouchAhead = 2;              // K-steps ahead of the stage refill
+  constexpr int kVmPerStep = kLoadsPerStep + kTouch;
+  const uint8_t* touch_ptr = A;
+  if constexpr (TOUCH) {
+    static_assert(BM == 256 && BN == 256 && kWaves == 4, "touch shares are laid out for the 256 x 256 tile");
+    const int idx = wave * 24 + (lane < 24 ? lane : 23);  // 0..95: 64 lines of A, then 32 of B
+    if (idx < 64) {
+      int r = m0 + (tile_n & 3) * 64 + idx;
+      r = r < M ? r : M - 1;
+      touch_ptr = A + (int64_t)r * lda;
+    } else {
+      int r = n0 + (tile_m & 7) * 32 + (idx - 64);
+      r = r < N ? r : N - 1;
+      touch_ptr = B + (int64_t)r * ldb;
+    }
+  }
+  auto touch = [&](int step) {
+    if constexpr (TOUCH) {
+      const int kt = step < k_steps ? step : k_steps - 1;
+      const uint8_t* p = touch_ptr + (uint32_t)kt * kBK;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+                   :
+                   : "s"(lds_base + (uint32_t)(NST * kStageBytes)), "v"(p)
+                   : "memory");
+    }
+  };
 
   v4f acc[TM][TN];
 #pragma unroll
@@ -225,7 +259,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   constexpr std::integral_constant<int, H> kHi{};
 #pragma unroll
   for (int p = 0; p < NST; ++p) fetch(p < k_steps ? p : k_steps - 1, (uint32_t)(p * kStageBytes));
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 1) * kLoadsPerStep) : "memory");
+#pragma unroll
+  for (int p = 0; p < kTouchAhead; ++p) touch(NST + p);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 1) * kLoadsPerStep + kTouchAhead * kTouch) : "memory");
   __syncthreads();
   const int a_row0 = wm * WM, b_row0 = wn * WN;
   // only the wave's first row differs between waves: fold it into the per-lane bases
@@ -316,7 +352,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
       }
     });
     // every fragment of this step has been requested; once they are in, the slot is free
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_waitcnt vmcnt(%0)" ::"n"((NST - 2) * kLoadsPerStep) : "memory");
+    // (the queue holds, in issue order, per step in flight its stage loads and then its touch
+    // load: all but the loads of step ks+1 and whatever precedes them may stay outstanding)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_waitcnt vmcnt(%0)" ::"n"((NST - 2) * kVmPerStep + kTouch) : "memory");
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     // ---- behind the bar: (hi,hi) reloads a[lo], (hi,lo) reloads b[hi], both from step ks+1
@@ -349,6 +387,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     });
 #pragma unroll
     for (int t = 0; t < kLoadsPerStep; ++t) dma();
+    touch(ks + NST + kTouchAhead);
   } while (++ks < k_steps);
   // the clamped refills of the last steps may still be landing: the epilogue reuses the LDS
   // (the no-ops cover the distance an assembly-written MFMA needs before its result is read)
@@ -392,18 +431,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4, bool TOUCH>
 int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N,
                 int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream) {
   const int tiles_m = (int)ceil_div(M, BM), tiles_n = (int)ceil_div(N, BN);
   // NST K-steps: panels + scale slots (1 KiB per operand and 128-element chunk of the step)
   size_t lds_bytes = (size_t)NST * (((BM + BN) / kGroupRows) * kGroupStride + 2048 * (FP4 ? 2 : 1));
   const size_t epi_bytes = (size_t)WAVES_M * WAVES_N * (BM / WAVES_M) * ((BN / WAVES_N) * 2 + 16);  // epilogue staging
+  if (TOUCH) lds_bytes += 256;  // dump area of the L2 prefetch loads
   if (lds_bytes < epi_bytes) lds_bytes = epi_bytes;
   // A grid that fits the chip once should land one workgroup per CU: asking for more than half
   // of the LDS keeps the dispatcher from pairing two workgroups on one CU while others idle.
   if ((int64_t)tiles_m * tiles_n <= device_facts().cu_count && lds_bytes < 82 * 1024) lds_bytes = 82 * 1024;
-  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST, FP4>;
+  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST, FP4, TOUCH>;
   if (lds_bytes > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess)
@@ -434,10 +474,11 @@ int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb
   hipStream_t s = as_hip(stream);
   const int variant = tuning("gemm.variant");
   const int64_t tiles256 = ceil_div(M, 256) * ceil_div(N, 256);
-  const bool big = variant == 2 || (variant == 0 && tiles256 >= device_facts().cu_count / 2);
+  const bool big = variant == 2 || variant == 7 || (variant == 0 && tiles256 >= device_facts().cu_count / 2);
   // <tile M, tile N, waves M, waves N, LDS ring slots, e2m1 operands>
-  if (big) return launch_gemm<256, 256, 2, 2, 2, FP4>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
-  return launch_gemm<128, 128, 2, 2, 4, FP4>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  if (big && variant == 7) return launch_gemm<256, 256, 2, 2, 2, FP4, false>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  if (big) return launch_gemm<256, 256, 2, 2, 2, FP4, true>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  return launch_gemm<128, 128, 2, 2, 4, FP4, false>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
 }
 
 }  // namespace dt
