@@ -20,6 +20,7 @@ Knob g_knobs[] = {
     {"cast.blocks_per_cu", 2},
     {"cast.pair_blocks_per_cu", 3},
     {"mx.blocks_per_cu", 16},
+    {"mx.col_blocks_per_cu", 16},
     {"gemm.variant", 0},
 };
 constexpr int kNumKnobs = sizeof(g_knobs) / sizeof(g_knobs[0]);

@@ -39,10 +39,14 @@ int launch_mx(const MxArgs& a) {
   }
   if (a.axis == 0 && !a.transpose && x_vec && a.cols % kV == 0 && aligned(a.data, 16) && aligned(a.scale, 8) &&
       a.rows < (1ll << 31) && a.cols < (1ll << 31) && LAYOUT == DT_SCALE_PLAIN) {
-    const int64_t row_tiles = a.rows / 32, col_tiles = ceil_div(a.cols, (int64_t)kWave * kV);
-    const unsigned grid = (unsigned)ceil_div(row_tiles * col_tiles, kBlock / kWave);
-    mx_col_kernel<IN, OUT><<<grid, kBlock, 0, a.stream>>>(a.x, (uint32_t)a.rows, (uint32_t)a.cols, a.data, a.scale);
-    return launch_status();
+    const int64_t tiles = (a.rows / 32) * ceil_div(a.cols, (int64_t)kWave * kV);
+    if (tiles <= 0x7FFFFFFFll) {
+      int64_t grid = (int64_t)cus * tuning("mx.col_blocks_per_cu");
+      if (grid > tiles) grid = tiles;
+      mx_col_kernel<IN, OUT><<<(unsigned)grid, kBlock, 0, a.stream>>>(a.x, (uint32_t)a.rows, (uint32_t)a.cols, a.data,
+                                                                     a.scale, (uint32_t)tiles);
+      return launch_status();
+    }
   }
   // general orientation / alignment
   int64_t outer, inner_blocks, xos, xes, dos, des, s_rows, s_cols;

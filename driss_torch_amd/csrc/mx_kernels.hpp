@@ -4,8 +4,8 @@
 //                  input, 8 elements per 16-byte load) or 8 lanes (fp32 input); the block
 //                  maximum is an integer max over DPP quad/row permutes -- no LDS.
 //  mx_col_kernel   blocks down columns, payload in the input orientation.  A lane owns 8
-//                  (fp32: 4) adjacent columns of a 32-row tile, so the block maximum needs
-//                  no cross-lane traffic at all.
+//                  (fp32: 4) adjacent columns x 8 rows; the four waves of a workgroup cover
+//                  a 32-row tile and merge their column maxima through LDS.
 //  mx_col_t_kernel blocks down columns, payload transposed through LDS so that the stores
 //                  are full 128-byte rows of the [cols, rows] output.
 //  mx_any_kernel   one thread per block, arbitrary strides: covers every (axis, transpose)
@@ -164,96 +164,135 @@ __global__ __launch_bounds__(kBlock) void mx_row_kernel(const void* __restrict__
 }
 
 // --------------------------------------------------------------- blocks down columns
-// In-place payload: one wave owns a 32-row tile of 64*kV columns; a lane holds kV adjacent
-// columns x 32 rows in registers.  Payload [rows, cols], scales [rows/32, cols].
+// In-place payload [rows, cols], scales [rows/32, cols].  A workgroup works on tiles of 32 rows x
+// 64*kV columns; wave w takes rows 8w..8w+7 of the tile, a lane kV adjacent columns x 8 rows
+// (eight 16-byte loads).  Every load instruction of a wave then reads one contiguous run of a
+// single row and a wave touches 8 rows, not 32: a read-only probe of this access pattern runs
+// at 5.9 TB/s against 5.0-5.4 TB/s for a wave that walks down 32 rows.  The four partial
+// column maxima meet in LDS (16 bytes per lane: packed 16-bit magnitudes, or four fp32
+// magnitudes), every wave derives the same scales and converts its own rows.  Tiles walk along
+// the columns first, so a band of 32 rows is one contiguous stretch of memory on the input and
+// on the output side.  The grid is persistent and the loads of a workgroup's next tile are
+// issued before the current tile is converted, so that reads, conversion and writes of
+// different tiles overlap.
 template <int IN, int OUT>
 __global__ __launch_bounds__(kBlock) void mx_col_kernel(const void* __restrict__ x, uint32_t rows, uint32_t cols,
-                                                        uint8_t* __restrict__ data, uint8_t* __restrict__ scale) {
+                                                        uint8_t* __restrict__ data, uint8_t* __restrict__ scale,
+                                                        uint32_t ntiles) {
   constexpr int kV = InTraits<IN>::kVec;   // columns per lane
   constexpr int kW = kV / 4;               // fp8 words per lane and row: 2 or 1
-  const int lane = threadIdx.x % kWave;
-  const uint32_t row_tiles = rows / 32u;
+  constexpr int kB = InTraits<IN>::kBytes;
+  __shared__ u32x4 part[2][kBlock / kWave][kWave];
+  const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
   const uint32_t col_tiles = (cols + kWave * kV - 1) / (kWave * kV);
-  const uint32_t wave_id = (blockIdx.x * kBlock + threadIdx.x) / kWave;
-  if (wave_id >= row_tiles * col_tiles) return;  // whole wave leaves; no barrier in this kernel
-  // consecutive waves walk down the rows first so a workgroup covers adjacent row tiles
-  const uint32_t ct = wave_id / row_tiles, rb = wave_id - ct * row_tiles;
-  const uint32_t col0 = ct * (kWave * kV) + lane * kV;
-  if (col0 >= cols) return;  // cols % kV == 0, so a lane is either fully inside or outside
-  const uint32_t row_vecs = cols / kV;
-  const u32x4* v = static_cast<const u32x4*>(x);
-  const uint64_t vfirst = (uint64_t)rb * 32u * row_vecs + col0 / kV;
-  u32x4 w[32];
-#pragma unroll
-  for (int i = 0; i < 32; ++i) w[i] = ld_stream(v + vfirst + (uint64_t)i * row_vecs);
+  const uint64_t pitch = (uint64_t)cols * kB;
 
-  // per-column magnitude maxima
-  uint32_t cm[kV];
-  if constexpr (IN == DT_BF16) {
-    uint32_t p0 = 0, p1 = 0, p2 = 0, p3 = 0;
+  // cols % kV == 0, so a lane is either fully inside or outside; rows % 32 == 0
+  auto load_tile = [&](u32x4 (&v)[8], uint32_t t) {
+    const uint32_t tr = t / col_tiles, tc = t - tr * col_tiles;
+    const uint32_t col0 = tc * (kWave * kV) + lane * kV;
+    if (col0 < cols) {
+      const uint8_t* p = static_cast<const uint8_t*>(x) + (uint64_t)(tr * 32u + w * 8u) * pitch + (uint64_t)col0 * kB;
 #pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      p0 = pk_absmax16(p0, w[i].x); p1 = pk_absmax16(p1, w[i].y);
-      p2 = pk_absmax16(p2, w[i].z); p3 = pk_absmax16(p3, w[i].w);
-    }
-    cm[0] = p0 << 16; cm[1] = p0 & 0xFFFF0000u; cm[2] = p1 << 16; cm[3] = p1 & 0xFFFF0000u;
-    cm[4] = p2 << 16; cm[5] = p2 & 0xFFFF0000u; cm[6] = p3 << 16; cm[7] = p3 & 0xFFFF0000u;
-  } else if constexpr (IN == DT_F16) {
-#pragma unroll
-    for (int c = 0; c < 8; ++c) cm[c] = 0;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      float f[8];
-      unpack8<IN>(w[i], f);
-#pragma unroll
-      for (int c = 0; c < 8; ++c) cm[c] = umax(cm[c], absbits_f32(as_u32(f[c])));
-    }
-  } else {
-    cm[0] = cm[1] = cm[2] = cm[3] = 0;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      cm[0] = umax(cm[0], absbits_f32(w[i].x)); cm[1] = umax(cm[1], absbits_f32(w[i].y));
-      cm[2] = umax(cm[2], absbits_f32(w[i].z)); cm[3] = umax(cm[3], absbits_f32(w[i].w));
-    }
-  }
-  float mult[kV];
-  bool nanc[kV];
-  uint32_t byte_lo = 0, byte_hi = 0;  // the kV scale bytes packed in column order
-#pragma unroll
-  for (int c = 0; c < kV; ++c) {
-    const MxScale<OUT> s = mx_scale_from_absbits<OUT>(cm[c]);
-    mult[c] = s.mult;
-    nanc[c] = s.nan;
-    if (c < 4) byte_lo |= s.byte << (8 * c); else byte_hi |= s.byte << (8 * (c - 4));
-  }
-  auto elem = [&](int i, int c) -> float {
-    if constexpr (IN == DT_F32) {
-      return as_f32(c == 0 ? w[i].x : c == 1 ? w[i].y : c == 2 ? w[i].z : w[i].w);
+      for (int i = 0; i < 8; ++i) v[i] = ld_stream(reinterpret_cast<const u32x4*>(p + i * pitch));
     } else {
-      const uint32_t d = (c >> 1) == 0 ? w[i].x : (c >> 1) == 1 ? w[i].y : (c >> 1) == 2 ? w[i].z : w[i].w;
-      if constexpr (IN == DT_BF16) return (c & 1) ? bf16_hi(d) : bf16_lo(d);
-      else return (c & 1) ? f16_hi(d) : f16_lo(d);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = u32x4{0u, 0u, 0u, 0u};
     }
   };
-  uint8_t* drow = data + (uint64_t)rb * 32u * cols + col0;
+  auto process = [&](const u32x4 (&v)[8], uint32_t t, int buf) {
+    const uint32_t tr = t / col_tiles, tc = t - tr * col_tiles;
+    const uint32_t col0 = tc * (kWave * kV) + lane * kV;
+    // this wave's column maxima over its 8 rows
+    u32x4 pm = {0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int i = 0; i < 32; ++i) {
-    uint32_t r[kW];
-#pragma unroll
-    for (int q = 0; q < kW; ++q) {
-      r[q] = pack4_finite<OUT>(elem(i, 4 * q) * mult[4 * q], elem(i, 4 * q + 1) * mult[4 * q + 1],
-                               elem(i, 4 * q + 2) * mult[4 * q + 2], elem(i, 4 * q + 3) * mult[4 * q + 3]);
-      uint32_t nanmask = (nanc[4 * q] ? 0xFFu : 0u) | (nanc[4 * q + 1] ? 0xFF00u : 0u) |
-                         (nanc[4 * q + 2] ? 0xFF0000u : 0u) | (nanc[4 * q + 3] ? 0xFF000000u : 0u);
-      r[q] = (r[q] & ~nanmask) | (0x7F7F7F7Fu & nanmask);
+    for (int i = 0; i < 8; ++i) {
+      if constexpr (IN == DT_F32) {
+        pm.x = umax(pm.x, absbits_f32(v[i].x)); pm.y = umax(pm.y, absbits_f32(v[i].y));
+        pm.z = umax(pm.z, absbits_f32(v[i].z)); pm.w = umax(pm.w, absbits_f32(v[i].w));
+      } else {
+        pm.x = pk_absmax16(pm.x, v[i].x); pm.y = pk_absmax16(pm.y, v[i].y);
+        pm.z = pk_absmax16(pm.z, v[i].z); pm.w = pk_absmax16(pm.w, v[i].w);
+      }
     }
-    if constexpr (kW == 2) st_stream(reinterpret_cast<u32x2*>(drow + (uint64_t)i * cols), u32x2{r[0], r[1]});
-    else st_stream(reinterpret_cast<uint32_t*>(drow + (uint64_t)i * cols), r[0]);
+    part[buf][w][lane] = pm;
+    __syncthreads();
+#pragma unroll
+    for (int o = 1; o < kBlock / kWave; ++o) {
+      const u32x4 q = part[buf][(w + o) % (kBlock / kWave)][lane];
+      if constexpr (IN == DT_F32) {
+        pm.x = umax(pm.x, q.x); pm.y = umax(pm.y, q.y); pm.z = umax(pm.z, q.z); pm.w = umax(pm.w, q.w);
+      } else {
+        pm.x = pk_absmax16(pm.x, q.x); pm.y = pk_absmax16(pm.y, q.y);
+        pm.z = pk_absmax16(pm.z, q.z); pm.w = pk_absmax16(pm.w, q.w);
+      }
+    }
+    uint32_t cm[kV];  // fp32 magnitude bits of the column maxima
+    if constexpr (IN == DT_F32) {
+      cm[0] = pm.x; cm[1] = pm.y; cm[2] = pm.z; cm[3] = pm.w;
+    } else if constexpr (IN == DT_BF16) {
+      cm[0] = pm.x << 16; cm[1] = pm.x & 0xFFFF0000u; cm[2] = pm.y << 16; cm[3] = pm.y & 0xFFFF0000u;
+      cm[4] = pm.z << 16; cm[5] = pm.z & 0xFFFF0000u; cm[6] = pm.w << 16; cm[7] = pm.w & 0xFFFF0000u;
+    } else {  // the largest f16 magnitude pattern is the largest magnitude; widen it exactly
+      cm[0] = as_u32(f16_lo(pm.x)); cm[1] = as_u32(f16_hi(pm.x)); cm[2] = as_u32(f16_lo(pm.y)); cm[3] = as_u32(f16_hi(pm.y));
+      cm[4] = as_u32(f16_lo(pm.z)); cm[5] = as_u32(f16_hi(pm.z)); cm[6] = as_u32(f16_lo(pm.w)); cm[7] = as_u32(f16_hi(pm.w));
+    }
+    float mult[kV];
+    uint32_t nanmask[kW] = {};
+    uint32_t bytes[kW] = {};  // the kV scale bytes packed in column order
+#pragma unroll
+    for (int c = 0; c < kV; ++c) {
+      const MxScale<OUT> sc = mx_scale_from_absbits<OUT>(cm[c]);
+      mult[c] = sc.mult;
+      bytes[c / 4] |= sc.byte << (8 * (c % 4));
+      nanmask[c / 4] |= sc.nan ? (0xFFu << (8 * (c % 4))) : 0u;
+    }
+    if (col0 < cols) {
+      uint8_t* drow = data + (uint64_t)(tr * 32u + w * 8u) * cols + col0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float f[8];
+        if constexpr (IN == DT_F32) {
+          f[0] = as_f32(v[i].x); f[1] = as_f32(v[i].y); f[2] = as_f32(v[i].z); f[3] = as_f32(v[i].w);
+        } else {
+          unpack8<IN>(v[i], f);
+        }
+        uint32_t r[kW];
+#pragma unroll
+        for (int q = 0; q < kW; ++q) {
+          r[q] = pack4_finite<OUT>(f[4 * q] * mult[4 * q], f[4 * q + 1] * mult[4 * q + 1], f[4 * q + 2] * mult[4 * q + 2],
+                                   f[4 * q + 3] * mult[4 * q + 3]);
+          r[q] = (r[q] & ~nanmask[q]) | (0x7F7F7F7Fu & nanmask[q]);
+        }
+        if constexpr (kW == 2) st_stream(reinterpret_cast<u32x2*>(drow + (uint64_t)i * cols), u32x2{r[0], r[1]});
+        else st_stream(reinterpret_cast<uint32_t*>(drow + (uint64_t)i * cols), r[0]);
+      }
+      if (w == 0) {  // scales [rows/32, cols]: kV adjacent bytes
+        uint8_t* srow = scale + (uint64_t)tr * cols + col0;
+        if constexpr (kW == 2) *reinterpret_cast<u32x2*>(srow) = u32x2{bytes[0], bytes[1]};
+        else *reinterpret_cast<uint32_t*>(srow) = bytes[0];
+      }
+    }
+  };
+
+  // part[] alternates between iterations, so one barrier per tile is enough: a wave can be at
+  // most one barrier ahead of the slowest reader of the buffer it will write two tiles on
+  const uint32_t stride = gridDim.x;
+  uint32_t t = blockIdx.x;  // < ntiles
+  u32x4 va[8], vb[8];
+  load_tile(va, t);
+  for (;;) {
+    uint32_t tn = t + stride;
+    if (tn < ntiles) load_tile(vb, tn);
+    process(va, t, 0);
+    if (tn >= ntiles) break;
+    t = tn;
+    tn = t + stride;
+    if (tn < ntiles) load_tile(va, tn);
+    process(vb, t, 1);
+    if (tn >= ntiles) break;
+    t = tn;
   }
-  // scales [rows/32, cols]: kV adjacent bytes
-  uint8_t* srow = scale + (uint64_t)rb * cols + col0;
-  if constexpr (kW == 2) *reinterpret_cast<u32x2*>(srow) = u32x2{byte_lo, byte_hi};
-  else *reinterpret_cast<uint32_t*>(srow) = byte_lo;
 }
 
 // ------------------------------------------- blocks down columns, transposed payload
