@@ -68,6 +68,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extra", action="store_true", help="skip the per-kernel table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--gemm-only", action="store_true",
+                    help="run only the block-scaled GEMM rows of the per-kernel table (for profiling) and print them")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain device copies of 128 MiB (to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
@@ -85,6 +87,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     K, W = args.steps, args.warmup
+    if args.gemm_only:
+        print(json.dumps({"kernels": extra_kernels(torch, cabi, util, dev, K, W, gemm_only=True)}))
+        return
 
     # ------------------------------------------------------------ headline step: config 2
     R = C = 8192
@@ -180,7 +185,7 @@ def main():
     print(json.dumps(result))
 
 
-def extra_kernels(torch, cabi, util, dev, K, W):
+def extra_kernels(torch, cabi, util, dev, K, W, gemm_only=False):
     """Every other kernel of the path at its benchmark config: rotated (HBM) and hot-cache."""
     rows = []
 
@@ -207,41 +212,45 @@ def extra_kernels(torch, cabi, util, dev, K, W):
         g = torch.Generator(device=dev).manual_seed(77 + i)
         return torch.randn(shape, generator=g, device=dev, dtype=torch.float32).to(dtype)
 
-    n = 8192 * 8192
-    hbm_row("amax", "bf16 [8192,8192]", n * 2, lambda i: (rnd((8192, 8192), bf16, i), torch.empty(1, device=dev)),
-            lambda x, o: cabi.amax(x, o))
-    hbm_row("amax", "fp32 [8192,8192]", n * 4, lambda i: (rnd((8192, 8192), f32, i), torch.empty(1, device=dev)),
-            lambda x, o: cabi.amax(x, o))
-    for od, nm in ((e4, "e4m3fn"), (e5, "e5m2")):
-        hbm_row("saturated_cast", f"bf16 [8192,8192] -> {nm}", n * 3,
-                lambda i, od=od: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=od, device=dev)),
-                lambda x, o, od=od: cabi.saturated_cast(x, scale1, od, cabi.ROUND_BF16_SCALE_PRODUCT, o))
-    n1 = 4096 * 4096
-    hbm_row("saturated_cast", "config 1: bf16 [4096,4096] -> e4m3fn", n1 * 3,
-            lambda i: (rnd((4096, 4096), bf16, i), torch.empty((4096, 4096), dtype=e4, device=dev)),
-            lambda x, o: cabi.saturated_cast(x, scale1, e4, cabi.ROUND_BF16_SCALE_PRODUCT, o))
-    hbm_row("saturated_cast", "fp32 [8192,8192] -> e4m3fn", n * 5,
-            lambda i: (rnd((8192, 8192), f32, i), torch.empty((8192, 8192), dtype=e4, device=dev)),
-            lambda x, o: cabi.saturated_cast(x, scale1, e4, cabi.ROUND_F32, o))
-    nr = 16384 * 4096
-    for dt_, nm, b in ((f32, "fp32", 4), (bf16, "bf16", 2)):
-        hbm_row("dynamic_scaled_quant_rowwise", f"config 3: {nm} [16384,4096] -> e4m3fn", nr * (b + 1) + 16384 * 8,
-                lambda i, dt_=dt_: (rnd((16384, 4096), dt_, i), torch.empty((16384, 4096), dtype=e4, device=dev),
-                                    torch.empty((16384, 1), device=dev), torch.empty((16384, 1), device=dev)),
-                lambda x, o, a, s: cabi.dynamic_scaled_quant_rowwise(x, e4, o, a, s))
-    mxb = n * 2 + n + n // 32
-    hbm_row("mx_fp8_quantize rows", "config 4: bf16 [8192,8192], blocks along rows", mxb,
-            lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
-                       torch.empty((8192, 256), dtype=torch.uint8, device=dev)),
-            lambda x, dd, s: cabi.mx_fp8_quantize(x, 1, False, e4, cabi.SCALE_PLAIN, dd, s))
-    hbm_row("mx_fp8_quantize cols (transposed out)", "config 4: bf16 [8192,8192], blocks down columns", mxb,
-            lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
-                       torch.empty((8192, 256), dtype=torch.uint8, device=dev)),
-            lambda x, dd, s: cabi.mx_fp8_quantize(x, 0, True, e4, cabi.SCALE_PLAIN, dd, s))
-    hbm_row("mx_fp8_quantize cols (in place)", "config 4: bf16 [8192,8192], blocks down columns", mxb,
-            lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
-                       torch.empty((256, 8192), dtype=torch.uint8, device=dev)),
-            lambda x, dd, s: cabi.mx_fp8_quantize(x, 0, False, e4, cabi.SCALE_PLAIN, dd, s))
+    def hbm_rows():
+        n = 8192 * 8192
+        hbm_row("amax", "bf16 [8192,8192]", n * 2, lambda i: (rnd((8192, 8192), bf16, i), torch.empty(1, device=dev)),
+                lambda x, o: cabi.amax(x, o))
+        hbm_row("amax", "fp32 [8192,8192]", n * 4, lambda i: (rnd((8192, 8192), f32, i), torch.empty(1, device=dev)),
+                lambda x, o: cabi.amax(x, o))
+        for od, nm in ((e4, "e4m3fn"), (e5, "e5m2")):
+            hbm_row("saturated_cast", f"bf16 [8192,8192] -> {nm}", n * 3,
+                    lambda i, od=od: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=od, device=dev)),
+                    lambda x, o, od=od: cabi.saturated_cast(x, scale1, od, cabi.ROUND_BF16_SCALE_PRODUCT, o))
+        n1 = 4096 * 4096
+        hbm_row("saturated_cast", "config 1: bf16 [4096,4096] -> e4m3fn", n1 * 3,
+                lambda i: (rnd((4096, 4096), bf16, i), torch.empty((4096, 4096), dtype=e4, device=dev)),
+                lambda x, o: cabi.saturated_cast(x, scale1, e4, cabi.ROUND_BF16_SCALE_PRODUCT, o))
+        hbm_row("saturated_cast", "fp32 [8192,8192] -> e4m3fn", n * 5,
+                lambda i: (rnd((8192, 8192), f32, i), torch.empty((8192, 8192), dtype=e4, device=dev)),
+                lambda x, o: cabi.saturated_cast(x, scale1, e4, cabi.ROUND_F32, o))
+        nr = 16384 * 4096
+        for dt_, nm, b in ((f32, "fp32", 4), (bf16, "bf16", 2)):
+            hbm_row("dynamic_scaled_quant_rowwise", f"config 3: {nm} [16384,4096] -> e4m3fn", nr * (b + 1) + 16384 * 8,
+                    lambda i, dt_=dt_: (rnd((16384, 4096), dt_, i), torch.empty((16384, 4096), dtype=e4, device=dev),
+                                        torch.empty((16384, 1), device=dev), torch.empty((16384, 1), device=dev)),
+                    lambda x, o, a, s: cabi.dynamic_scaled_quant_rowwise(x, e4, o, a, s))
+        mxb = n * 2 + n + n // 32
+        hbm_row("mx_fp8_quantize rows", "config 4: bf16 [8192,8192], blocks along rows", mxb,
+                lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
+                           torch.empty((8192, 256), dtype=torch.uint8, device=dev)),
+                lambda x, dd, s: cabi.mx_fp8_quantize(x, 1, False, e4, cabi.SCALE_PLAIN, dd, s))
+        hbm_row("mx_fp8_quantize cols (transposed out)", "config 4: bf16 [8192,8192], blocks down columns", mxb,
+                lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
+                           torch.empty((8192, 256), dtype=torch.uint8, device=dev)),
+                lambda x, dd, s: cabi.mx_fp8_quantize(x, 0, True, e4, cabi.SCALE_PLAIN, dd, s))
+        hbm_row("mx_fp8_quantize cols (in place)", "config 4: bf16 [8192,8192], blocks down columns", mxb,
+                lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
+                           torch.empty((256, 8192), dtype=torch.uint8, device=dev)),
+                lambda x, dd, s: cabi.mx_fp8_quantize(x, 0, False, e4, cabi.SCALE_PLAIN, dd, s))
+
+    if not gemm_only:
+        hbm_rows()
 
     # MXFP8 GEMM, config 5
     M = N = Kd = 8192
