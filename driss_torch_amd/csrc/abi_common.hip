@@ -14,6 +14,8 @@ struct Knob {
   int value;
 };
 // Launch-shape knobs.  Workgroups per CU for the persistent grids, chosen on MI355X.
+//   gemm.variant: 0 = pick the tile by problem size, 1 = 128x128 tiles, 2 = 256x256 tiles,
+//                 7 = 256x256 tiles without the L2 prefetch loads
 Knob g_knobs[] = {
     {"amax.blocks_per_cu", 1},
     {"amax.stream_before_cast", 0},
