@@ -87,6 +87,8 @@ _workspaces = {}
 def workspace(device=None) -> torch.Tensor:
     """A zero-initialised reduction workspace for the current (device, stream)."""
     dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    if dev.index is None:  # "cuda" means the current device: same workspace as "cuda:<current>"
+        dev = torch.device("cuda", torch.cuda.current_device())
     key = (dev.index, _stream())
     ws = _workspaces.get(key)
     if ws is None:

@@ -14,6 +14,8 @@ struct Knob {
   int value;
 };
 // Launch-shape knobs.  Workgroups per CU for the persistent grids, chosen on MI355X.
+//   dynamic.resident: 1 = per-tensor dynamic quantization of a tensor that fits the chip runs as one
+//                 kernel that keeps it in registers and LDS; dynamic.resident_min_kib = smallest such tensor
 //   gemm.variant: 0 = pick the tile by problem size, 1 = 128x128 tiles, 2 = 256x256 tiles,
 //                 7 = 256x256 tiles without the L2 prefetch loads
 Knob g_knobs[] = {
@@ -24,6 +26,9 @@ Knob g_knobs[] = {
     {"mx.blocks_per_cu", 16},
     {"mx.col_blocks_per_cu", 16},
     {"gemm.variant", 0},
+    {"dynamic.resident", 1},
+    {"dynamic.resident_min_kib", 1024},
+    {"dynamic.resident_spin_limit", 1 << 19},
 };
 constexpr int kNumKnobs = sizeof(g_knobs) / sizeof(g_knobs[0]);
 
@@ -83,7 +88,7 @@ int dt_workspace_init(void* workspace, size_t workspace_bytes, dt_stream_t strea
   if (workspace_bytes < dt::kWsBytes) return DT_ERR_WORKSPACE;
   if (!dt::aligned(workspace, 256)) return DT_ERR_MISALIGNED;
   // a fill kernel rather than hipMemsetAsync, so the call is safe under graph capture
-  dt::zero_words_kernel<<<1, 64, 0, dt::as_hip(stream)>>>(static_cast<uint32_t*>(workspace), 64);
+  dt::zero_words_kernel<<<1, 128, 0, dt::as_hip(stream)>>>(static_cast<uint32_t*>(workspace), 128);
   return dt::launch_status();
 }
 

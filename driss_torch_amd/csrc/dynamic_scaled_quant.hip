@@ -1,10 +1,12 @@
 // dt_dynamic_scaled_quant*: amax -> scale -> saturating fp8 cast, per tensor and per row (C ABI).
 //
-// Per tensor the work is two stream-ordered kernels: the amax reduction, whose last
-// workgroup also derives the scale(s) into the workspace, and the streaming cast, which
-// reads the scale from there.  The second read of x is served from the memory-side cache
-// for tensors that fit it.
+// A tensor that fits the chip's registers and LDS (128 MiB on 256 CUs) goes through one kernel
+// that holds it there between the reduction and the cast (resident_kernels.hpp).  Otherwise
+// the work is two stream-ordered kernels: the amax reduction, whose last workgroup also derives
+// the scale(s) into the workspace, and the streaming cast, which reads the scale from there;
+// the second read of x is then served from the memory-side cache as far as it fits.
 #include "quant_kernels.hpp"
+#include "resident_kernels.hpp"
 #include "rowwise_kernels.hpp"
 
 namespace {
@@ -19,6 +21,9 @@ extern "C" int dt_dynamic_scaled_quant(const void* x, int in_dtype, int64_t nume
   if (int st = dt::check_workspace(workspace, workspace_bytes)) return st;
   hipStream_t s = dt::as_hip(stream);
   const float fm = fmax_of(out_dtype);
+  if (dt::launch_resident<false>(x, in_dtype, numel, out_dtype, round_mode, workspace, out, nullptr, amax_out, scale_out, fm,
+                                 0.f, s) == DT_OK)
+    return DT_OK;
   int st = in_dtype == DT_F32 ? dt::launch_amax<DT_F32>(x, numel, workspace, amax_out, scale_out, 1, fm, 0.f, s)
                               : dt::launch_amax<DT_BF16>(x, numel, workspace, amax_out, scale_out, 1, fm, 0.f, s);
   if (st) return st;
@@ -54,6 +59,10 @@ extern "C" int dt_dynamic_scaled_quant_pair(const void* x, int in_dtype, int64_t
                                             void* workspace, size_t workspace_bytes, dt_stream_t stream) {
   if (int st = dt::check_cast_args(x, in_dtype, numel, DT_E4M3FN, round_mode, out_e4m3fn)) return st;
   if (!out_e5m2) return DT_ERR_NULL_POINTER;
+  if (numel > 0 && dt::check_workspace(workspace, workspace_bytes) == DT_OK && (in_dtype == DT_F32 || in_dtype == DT_BF16) &&
+      dt::launch_resident<true>(x, in_dtype, numel, DT_E4M3FN, round_mode, workspace, out_e4m3fn, out_e5m2, amax_out,
+                                scale_out, 448.0f, 57344.0f, dt::as_hip(stream)) == DT_OK)
+    return DT_OK;
   if (int st = dt_amax_scales(x, in_dtype, numel, amax_out, scale_out, workspace, workspace_bytes, stream)) return st;
   const float* scale = reinterpret_cast<const float*>(static_cast<const uint8_t*>(workspace) + dt::kWsScale);
   return dt_saturated_cast_pair(x, in_dtype, numel, scale, round_mode, out_e4m3fn, out_e5m2, stream);

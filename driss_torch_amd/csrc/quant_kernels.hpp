@@ -161,11 +161,14 @@ inline int launch_amax(const void* x, int64_t numel, void* ws, float* amax_out, 
 // --------------------------------------------------------------------------- cast ----
 // ROUND_BF16: round the product to bf16 before the convert (modes 1 and 2 of
 // dt_round_mode, bf16 input only); ROUND_SCALE: also round the scale itself (mode 2).
-template <int IN, int OUT, bool ROUND_BF16>
+// CHECK_NAN = false is for callers that know no product can be a NaN (no NaN and no infinity in
+// the tensor, finite scale): the result is the same, without the test.
+template <int IN, int OUT, bool ROUND_BF16, bool CHECK_NAN = true>
 __device__ __forceinline__ void cast_vec(u32x4 w, float s, uint8_t* __restrict__ out, int64_t vec_index) {
   if constexpr (IN == DT_F32) {
     const float p0 = as_f32(w.x) * s, p1 = as_f32(w.y) * s, p2 = as_f32(w.z) * s, p3 = as_f32(w.w) * s;
-    st_stream(reinterpret_cast<uint32_t*>(out) + vec_index, pack4<OUT>(p0, p1, p2, p3));
+    st_stream(reinterpret_cast<uint32_t*>(out) + vec_index,
+              CHECK_NAN ? pack4<OUT>(p0, p1, p2, p3) : pack4_clamped<OUT>(p0, p1, p2, p3));
   } else {
     float p[8] = {bf16_lo(w.x) * s, bf16_hi(w.x) * s, bf16_lo(w.y) * s, bf16_hi(w.y) * s,
                   bf16_lo(w.z) * s, bf16_hi(w.z) * s, bf16_lo(w.w) * s, bf16_hi(w.w) * s};
@@ -178,7 +181,7 @@ __device__ __forceinline__ void cast_vec(u32x4 w, float s, uint8_t* __restrict__
     r.y = pack4_clamped<OUT>(p[4], p[5], p[6], p[7]);
     const bool any_nan = (p[0] != p[0]) | (p[1] != p[1]) | (p[2] != p[2]) | (p[3] != p[3]) | (p[4] != p[4]) |
                          (p[5] != p[5]) | (p[6] != p[6]) | (p[7] != p[7]);
-    if (__builtin_expect(any_nan, 0)) {
+    if (CHECK_NAN && __builtin_expect(any_nan, 0)) {
       r.x = nan_patch4(r.x, p[0], p[1], p[2], p[3]);
       r.y = nan_patch4(r.y, p[4], p[5], p[6], p[7]);
     }

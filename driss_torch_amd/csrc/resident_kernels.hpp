@@ -1,0 +1,355 @@
+// Per-tensor dynamic quantization with the tensor held on the chip between its two passes.
+//
+// amax -> scale -> cast needs x twice, and the second pass cannot start before the first has
+// finished everywhere.  An MI355X has 256 CUs x (512 KB of vector registers + 160 KB of LDS):
+// a tensor of up to 128 MiB fits into the registers and the LDS of one workgroup per CU.  So one
+// persistent workgroup per CU loads its share of x once (16-byte vectors, grid-strided: 96 per
+// lane stay in registers, 36 more go to LDS), reduces |x| on the way, meets the other workgroups
+// at a grid-wide barrier built on the reduction's own atomics, derives the scale(s) and converts
+// straight out of registers and LDS.  HBM sees one read of x and the fp8 writes; the two-kernel
+// path reads x from HBM and again from the memory-side cache.  Measured on 8192 x 8192 bf16 ->
+// e4m3fn + e5m2: 65 us for the two kernels, see bench.py for this one.
+//
+// The barrier needs every workgroup of the grid to be resident at once.  The grid is at most one
+// workgroup per CU and a workgroup owns a CU's whole register file, so the dispatcher spreads
+// the grid one per CU; other kernels only delay that.  (hipLaunchCooperativeKernel would check
+// it, but costs 18 us per launch here, more than the kernel saves.)  What must not happen is two
+// such grids at once, so the host chains them.  The wait is bounded all the same: a workgroup
+// that gives up sets a sticky flag in the workspace and writes NaN, and every wave reaches the
+// end of the kernel whatever happens.
+#pragma once
+
+#include <mutex>
+
+#include "quant_kernels.hpp"
+
+namespace dt {
+
+constexpr int kResRegVecs = 92;   // 16-byte vectors per lane kept in registers (368 VGPRs)
+constexpr int kResLdsVecs = 36;   // ... and in LDS (144 KiB per workgroup)
+constexpr int kResVecs = kResRegVecs + kResLdsVecs;
+constexpr size_t kResLdsBytes = (size_t)kResLdsVecs * kBlock * 16;
+constexpr size_t kWsDepart = 192;  // u32 departure counter of the grid barrier, zero between launches
+constexpr size_t kWsRelease = 256; // u64 release word of the grid barrier (a cache line of its own), zero between launches
+constexpr size_t kWsTimeout = 196; // u32, set (and left set) if a barrier wait ever gave up
+
+// One vector to e4m3fn and e5m2 at once, for products that cannot be NaN.  The two scales are
+// fmax / amax with fmax = 448 and 57344 = 128 * 448, so scale_e5m2 == 128 * scale_e4m3 exactly
+// (a power of two commutes with every rounding on the way, also with the bf16 roundings of
+// modes 1 and 2, and with the clamp): the e5m2 operand is the clamped e4m3 operand times 128.
+template <int IN, bool ROUND_BF16>
+__device__ __forceinline__ void cast_vec_pair_finite(u32x4 w, float s4, uint8_t* __restrict__ out4,
+                                                     uint8_t* __restrict__ out5, uint32_t vec_index) {
+  constexpr int kV = InTraits<IN>::kVec;
+  float p[kV];
+  if constexpr (IN == DT_F32) {
+    p[0] = as_f32(w.x) * s4; p[1] = as_f32(w.y) * s4; p[2] = as_f32(w.z) * s4; p[3] = as_f32(w.w) * s4;
+  } else {
+    p[0] = bf16_lo(w.x) * s4; p[1] = bf16_hi(w.x) * s4; p[2] = bf16_lo(w.y) * s4; p[3] = bf16_hi(w.y) * s4;
+    p[4] = bf16_lo(w.z) * s4; p[5] = bf16_hi(w.z) * s4; p[6] = bf16_lo(w.w) * s4; p[7] = bf16_hi(w.w) * s4;
+    if constexpr (ROUND_BF16) {
+      round2_to_bf16(p[0], p[1]); round2_to_bf16(p[2], p[3]);
+      round2_to_bf16(p[4], p[5]); round2_to_bf16(p[6], p[7]);
+    }
+  }
+  uint32_t r4[kV / 4], r5[kV / 4];
+#pragma unroll
+  for (int q = 0; q < kV / 4; ++q) {
+    const float c0 = clamp_fp8<DT_E4M3FN>(p[4 * q]), c1 = clamp_fp8<DT_E4M3FN>(p[4 * q + 1]);
+    const float c2 = clamp_fp8<DT_E4M3FN>(p[4 * q + 2]), c3 = clamp_fp8<DT_E4M3FN>(p[4 * q + 3]);
+    r4[q] = cvt_pk<DT_E4M3FN, true>(c2, c3, cvt_pk<DT_E4M3FN, false>(c0, c1, 0u));
+    r5[q] = cvt_pk<DT_E5M2, true>(c2 * 128.0f, c3 * 128.0f, cvt_pk<DT_E5M2, false>(c0 * 128.0f, c1 * 128.0f, 0u));
+  }
+  if constexpr (IN == DT_F32) {
+    st_stream(reinterpret_cast<uint32_t*>(out4) + vec_index, r4[0]);
+    st_stream(reinterpret_cast<uint32_t*>(out5) + vec_index, r5[0]);
+  } else {
+    st_stream(reinterpret_cast<u32x2*>(out4) + vec_index, u32x2{r4[0], r4[1]});
+    st_stream(reinterpret_cast<u32x2*>(out5) + vec_index, u32x2{r5[0], r5[1]});
+  }
+}
+
+template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR>
+__global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __restrict__ x, int64_t nvec, int tail,
+                                                               uint8_t* __restrict__ ws, uint8_t* __restrict__ out,
+                                                               uint8_t* __restrict__ out2, float* __restrict__ amax_out,
+                                                               float* __restrict__ scale_out, float fmax0, float fmax1,
+                                                               uint32_t spin_limit) {
+  constexpr int kV = InTraits<IN>::kVec;
+  constexpr int OUT2 = OUT == DT_E4M3FN ? DT_E5M2 : DT_E4M3FN;
+  extern __shared__ __attribute__((aligned(16))) u32x4 keep[];  // [kResLdsVecs][kBlock]
+  __shared__ uint32_t red[kBlock / kWave];
+  __shared__ uint32_t bcast;
+  const int tid = threadIdx.x;
+  const u32x4* v = static_cast<const u32x4*>(x);
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  const int64_t first = (int64_t)blockIdx.x * kBlock + tid;
+
+  // ---- pass 1: load the share once, keep it, reduce |x|
+  u32x4 r[kResRegVecs];
+  uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+  // Loads are issued in batches of kResBatch before any of them is looked at (one wave per SIMD:
+  // nothing else keeps the memory system busy while a wave waits).  No branch around a load
+  // either: past the end the last vector is read again and replaced by zeros.
+  auto fetch = [&](int k) -> u32x4 {
+    const int64_t i = first + k * stride;
+    return ld_stream(v + (i < nvec ? i : nvec - 1));
+  };
+  auto absorb = [&](int k, u32x4& w) {
+    const bool inside = first + k * stride < nvec;
+    w.x = inside ? w.x : 0u; w.y = inside ? w.y : 0u; w.z = inside ? w.z : 0u; w.w = inside ? w.w : 0u;
+    if constexpr (IN == DT_F32) {
+      a0 = umax(a0, absbits_f32(w.x)); a1 = umax(a1, absbits_f32(w.y));
+      a2 = umax(a2, absbits_f32(w.z)); a3 = umax(a3, absbits_f32(w.w));
+    } else {
+      a0 = pk_absmax16(a0, w.x); a1 = pk_absmax16(a1, w.y);
+      a2 = pk_absmax16(a2, w.z); a3 = pk_absmax16(a3, w.w);
+    }
+  };
+  constexpr int kResBatch = 16;
+  static_assert(kResRegVecs % 4 == 0 && kResLdsVecs % 4 == 0, "batches");
+  // the LDS part first (through a batch of registers), then the register part in place
+#pragma unroll
+  for (int b = 0; b < kResLdsVecs; b += kResBatch) {
+    u32x4 t[kResBatch];
+#pragma unroll
+    for (int j = 0; j < kResBatch; ++j)
+      if (b + j < kResLdsVecs) t[j] = fetch(kResRegVecs + b + j);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < kResBatch; ++j)
+      if (b + j < kResLdsVecs) {
+        absorb(kResRegVecs + b + j, t[j]);
+        keep[(b + j) * kBlock + tid] = t[j];
+      }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int b = 0; b < kResRegVecs; b += kResBatch) {
+#pragma unroll
+    for (int j = 0; j < kResBatch; ++j)
+      if (b + j < kResRegVecs) r[b + j] = fetch(b + j);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < kResBatch; ++j)
+      if (b + j < kResRegVecs) absorb(b + j, r[b + j]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  uint32_t m;
+  if constexpr (IN == DT_F32) {
+    m = umax(umax(a0, a1), umax(a2, a3));
+  } else {
+    uint32_t p = pk_absmax16(pk_absmax16(a0, a1), pk_absmax16(a2, a3));
+    m = umax(p & 0xFFFFu, p >> 16) << 16;
+  }
+  if (blockIdx.x == 0 && tid < tail) m = umax(m, absbits_of<IN>(x, nvec * kV + tid));  // x is 16-byte aligned: no head
+  m = block_umax<kBlock / kWave>(m, red);
+
+  // ---- grid barrier on the reduction's atomics: fold the partial into the running maximum,
+  // take a ticket, wait until every workgroup has taken one, read the maximum.  The last
+  // workgroup to leave publishes amax and the scales and re-arms the workspace.
+  // The waiting workgroups poll a word of its own (another cache line): polling the line the
+  // arrivals update slows those atomics down for everybody (measured: 8 us -> see bench).
+  uint32_t* running = reinterpret_cast<uint32_t*>(ws + kWsRunning);
+  uint32_t* ticket = reinterpret_cast<uint32_t*>(ws + kWsTicket);
+  uint32_t* depart = reinterpret_cast<uint32_t*>(ws + kWsDepart);
+  uint64_t* release = reinterpret_cast<uint64_t*>(ws + kWsRelease);  // (1 << 32) | amax bits once everybody has arrived
+  if (tid == 0) {
+    uint32_t before = __hip_atomic_fetch_max(running, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t one = 1u;  // the ticket depends on the returned value, so the two atomics stay ordered
+    asm volatile("v_and_or_b32 %0, %1, 0, %0" : "+v"(one) : "v"(before));
+    const uint32_t t = __hip_atomic_fetch_add(ticket, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t bits;
+    if (t == gridDim.x - 1) {
+      // last to arrive: every other workgroup's maximum was folded in before it took its ticket
+      bits = __hip_atomic_load(running, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(release, (1ull << 32) | bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+      uint32_t spins = 0;
+      uint64_t rel;
+      while (((rel = __hip_atomic_load(release, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) == 0) {
+        __builtin_amdgcn_s_sleep(2);
+        if (++spins >= spin_limit) {  // cannot happen when the grid is resident; never hang the GPU
+          __hip_atomic_store(reinterpret_cast<uint32_t*>(ws + kWsTimeout), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          rel = 0x7FC00000ull;  // the outputs of this workgroup become NaN: a loud failure
+          break;
+        }
+      }
+      bits = (uint32_t)rel;
+    }
+    bcast = bits;
+    uint32_t dep = 1u;
+    asm volatile("v_and_or_b32 %0, %1, 0, %0" : "+v"(dep) : "v"(bits));  // leave only after the read
+    if (__hip_atomic_fetch_add(depart, dep, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1) {
+      __hip_atomic_store(running, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(depart, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(release, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const float amax = as_f32(bits);
+      float* wscale = reinterpret_cast<float*>(ws + kWsScale);
+      *reinterpret_cast<float*>(ws + kWsAmax) = amax;
+      if (amax_out) *amax_out = amax;
+      const float s0 = amax_to_scale(amax, fmax0);
+      wscale[0] = s0;
+      if (scale_out) scale_out[0] = s0;
+      if constexpr (PAIR) {
+        const float s1 = amax_to_scale(amax, fmax1);
+        wscale[1] = s1;
+        if (scale_out) scale_out[1] = s1;
+      }
+    }
+  }
+  __syncthreads();
+  const float amax = as_f32(bcast);
+  float s = amax_to_scale(amax, fmax0), s2 = PAIR ? amax_to_scale(amax, fmax1) : 0.f;
+  if constexpr (ROUND_SCALE) { s = round_to_bf16(s); s2 = round_to_bf16(s2); }
+
+  // ---- pass 2: convert out of registers and LDS.  A product can only be a NaN if the tensor
+  // holds a NaN or an infinity (inf * 0), which amax tells: then x is simply read again by the
+  // streaming cast with its NaN handling (a rare path, and the only one with a function call,
+  // which must not sit among 368 live registers).  Otherwise no test is needed at all.
+  if (bcast >= 0x7F800000u) {
+    for (int64_t i = first; i < nvec; i += stride) {
+      const u32x4 w = ld_stream(v + i);
+      cast_vec<IN, OUT, ROUND_BF16>(w, s, out, i);
+      if constexpr (PAIR) cast_vec<IN, OUT2, ROUND_BF16>(w, s2, out2, i);
+    }
+  } else {
+    // The vector indices are recomputed from an opaque copy of the first one: reusing pass 1's
+    // 128 index pairs would keep them in registers across the barrier, next to the data.
+    // (at most 2^31 vectors fit the chip, so 32-bit indices do)
+    uint32_t first2 = (uint32_t)first;
+    asm volatile("" : "+v"(first2));
+    const uint32_t stride32 = (uint32_t)stride, nvec32 = (uint32_t)nvec;
+    auto emit = [&](int k, u32x4 w) {
+      const uint32_t i = first2 + k * stride32;
+      if (i < nvec32) {
+        if constexpr (PAIR) {
+          static_assert(!PAIR || OUT == DT_E4M3FN, "the pair is e4m3fn + e5m2");
+          cast_vec_pair_finite<IN, ROUND_BF16>(w, s, out, out2, i);
+        } else {
+          cast_vec<IN, OUT, ROUND_BF16, false>(w, s, out, i);
+        }
+      }
+    };
+#pragma unroll
+    for (int k = 0; k < kResRegVecs; ++k) emit(k, r[k]);
+#pragma unroll
+    for (int k = 0; k < kResLdsVecs; ++k) emit(kResRegVecs + k, keep[k * kBlock + tid]);
+  }
+  if (blockIdx.x == 0 && tid < tail) {
+    const int64_t e = nvec * kV + tid;
+    out[e] = cast_one<IN, OUT, ROUND_BF16>(x, e, s);
+    if constexpr (PAIR) out2[e] = cast_one<IN, OUT2, ROUND_BF16>(x, e, s2);
+  }
+}
+
+// Host-side chaining of resident launches (see launch_resident_impl).
+struct ResidentGate {
+  static constexpr int kMaxDevices = 16;
+  std::mutex mu;
+  bool used[kMaxDevices] = {};
+  hipStream_t last_stream[kMaxDevices] = {};  // stream of the device's latest resident launch
+  hipEvent_t event[kMaxDevices] = {};         // recorded there when a launch arrives on another stream
+};
+inline ResidentGate& resident_gate() {
+  static ResidentGate* g = new ResidentGate();  // leaked on purpose: no HIP calls at process exit
+  return *g;
+}
+
+// Launch the resident kernel if the tensor qualifies.  Returns DT_OK when it was launched, a
+// negative value when the caller should take the two-kernel path instead.
+constexpr int kResidentNotTaken = -1;
+template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR>
+inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* out, void* out2, float* amax_out,
+                                float* scale_out, float fmax0, float fmax1, hipStream_t stream) {
+  if constexpr (PAIR && OUT != DT_E4M3FN) return kResidentNotTaken;  // the pair is (e4m3fn, e5m2)
+  else {
+  constexpr int kV = InTraits<IN>::kVec;
+  constexpr size_t kStoreAlign = IN == DT_F32 ? 4 : 8;
+  if (!aligned(x, 16) || !aligned(out, kStoreAlign) || (PAIR && !aligned(out2, kStoreAlign))) return kResidentNotTaken;
+  const int cus = device_facts().cu_count;
+  int64_t nvec = numel / kV;
+  int tail = (int)(numel % kV);
+  if (nvec < 1 || nvec > (int64_t)cus * kBlock * kResVecs) return kResidentNotTaken;
+  int64_t grid = ceil_div(nvec, (int64_t)kBlock * 4);  // at least 4 vectors per lane before another workgroup joins
+  if (grid > cus) grid = cus;
+  if (grid < 1) grid = 1;
+  auto kernel = resident_quant_kernel<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR>;
+  static bool configured = false;  // per instantiation; the attribute is idempotent, a race only repeats the call
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)kResLdsBytes) != hipSuccess) {
+      (void)hipGetLastError();
+      return kResidentNotTaken;
+    }
+    configured = true;
+  }
+  uint8_t* w = static_cast<uint8_t*>(ws);
+  uint8_t* o = static_cast<uint8_t*>(out);
+  uint8_t* o2 = static_cast<uint8_t*>(out2);
+  const uint32_t spin_limit = (uint32_t)tuning("dynamic.resident_spin_limit");
+  // Two grids of this kernel in flight at once (two streams) could each hold part of the chip
+  // and wait for the rest for ever: resident launches of a device are chained: one that arrives
+  // on another stream than the previous one first waits for that stream's tail.  A stream under graph capture cannot take such a dependency.
+  ResidentGate& gate = resident_gate();
+  std::lock_guard<std::mutex> lock(gate.mu);
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return kResidentNotTaken;
+  }
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  if (dev < 0 || dev >= ResidentGate::kMaxDevices) return kResidentNotTaken;
+  if (gate.used[dev] && gate.last_stream[dev] != stream) {
+    // mark the tail of the stream that ran the previous resident kernel and wait for it here
+    if (!gate.event[dev] && hipEventCreateWithFlags(&gate.event[dev], hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      gate.event[dev] = nullptr;
+      return kResidentNotTaken;
+    }
+    if (hipEventRecord(gate.event[dev], gate.last_stream[dev]) != hipSuccess) {
+      (void)hipGetLastError();           // that stream is gone: its work may still be running
+      (void)hipDeviceSynchronize();
+    } else if (hipStreamWaitEvent(stream, gate.event[dev], 0) != hipSuccess) {
+      (void)hipGetLastError();
+      return kResidentNotTaken;
+    }
+  }
+  kernel<<<(unsigned)grid, kBlock, kResLdsBytes, stream>>>(x, nvec, tail, w, o, o2, amax_out, scale_out, fmax0, fmax1,
+                                                         spin_limit);
+  const int st = launch_status();
+  if (st == DT_OK) {
+    gate.used[dev] = true;
+    gate.last_stream[dev] = stream;
+  }
+  return st;
+  }
+}
+
+template <bool PAIR>
+inline int launch_resident(const void* x, int in_dtype, int64_t numel, int out_dtype, int round_mode, void* ws, void* out,
+                           void* out2, float* amax_out, float* scale_out, float fmax0, float fmax1, hipStream_t stream) {
+  if (!tuning("dynamic.resident") || numel * (in_dtype == DT_F32 ? 4 : 2) < (int64_t)tuning("dynamic.resident_min_kib") * 1024)
+    return kResidentNotTaken;
+#define DT_RES(IN, OUT, RB, RS) \
+  return launch_resident_impl<IN, OUT, RB, RS, PAIR>(x, numel, ws, out, out2, amax_out, scale_out, fmax0, fmax1, stream)
+  if (in_dtype == DT_F32) {
+    if (out_dtype == DT_E4M3FN) DT_RES(DT_F32, DT_E4M3FN, false, false);
+    DT_RES(DT_F32, DT_E5M2, false, false);
+  }
+  if (round_mode == DT_ROUND_F32) {
+    if (out_dtype == DT_E4M3FN) DT_RES(DT_BF16, DT_E4M3FN, false, false);
+    DT_RES(DT_BF16, DT_E5M2, false, false);
+  }
+  if (round_mode == DT_ROUND_BF16_PRODUCT) {
+    if (out_dtype == DT_E4M3FN) DT_RES(DT_BF16, DT_E4M3FN, true, false);
+    DT_RES(DT_BF16, DT_E5M2, true, false);
+  }
+  if (out_dtype == DT_E4M3FN) DT_RES(DT_BF16, DT_E4M3FN, true, true);
+  DT_RES(DT_BF16, DT_E5M2, true, true);
+#undef DT_RES
+}
+
+}  // namespace dt

@@ -1,0 +1,161 @@
+"""GPU parity of the single-kernel ("resident") per-tensor dynamic quantization: the tensor is held
+in registers and LDS between the amax reduction and the cast.  Bit for bit against the CPU oracle
+and against the two-kernel path, on ragged sizes, at and past the capacity of the chip, with NaN and
+infinity in the data, from two streams, and with the barrier's wait forced to give up."""
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+MODE = {1: "ROUND_V1", 2: "ROUND_V2", 3: "ROUND_V3"}
+
+
+@pytest.fixture()
+def cabi(gpu_device):
+    from driss_torch_amd import cabi as c
+
+    keep = {k: c.get_tuning(k) for k in ("dynamic.resident", "dynamic.resident_min_kib", "dynamic.resident_spin_limit")}
+    c.set_tuning("dynamic.resident_min_kib", 0)  # every size takes the resident kernel
+    yield c
+    for k, v in keep.items():
+        c.set_tuning(k, v)
+
+
+def _timeout_flag(cabi):
+    ws = cabi.workspace(torch.device("cuda"))
+    torch.cuda.synchronize()
+    return int(ws[196:200].cpu().view(torch.int32).item())
+
+
+def _both_paths(cabi, x, fn):
+    cabi.set_tuning("dynamic.resident", 1)
+    a = fn(x)
+    cabi.set_tuning("dynamic.resident", 0)
+    b = fn(x)
+    cabi.set_tuning("dynamic.resident", 1)
+    return a, b
+
+
+@pytest.mark.parametrize("shape", [(1, 8), (3, 7), (64, 17), (512, 127), (1000, 1003), (4096, 4097), (1, 1 << 20)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("fp8_dtype", [E4, E5])
+def test_resident_single_output(cabi, shape, in_dtype, fp8_dtype):
+    x = util.normal_with_outliers(shape, 31 + shape[1], in_dtype)
+    modes = (1, 2, 3) if in_dtype == torch.bfloat16 else (3,)
+    for mode in modes:
+        (out, amax, scale), (out2, amax2, scale2) = _both_paths(cabi, x.cuda(), lambda t: cabi.dynamic_scaled_quant(t, fp8_dtype, mode))
+        ref, ramax, rscale = co.dynamic_scaled_quant(x, fp8_dtype, getattr(co, MODE[mode]))
+        assert torch.equal(util.codes(out), ref) and torch.equal(util.codes(out2), ref)
+        assert amax.item() == ramax.item() == amax2.item() and scale.item() == rscale.item() == scale2.item()
+    assert _timeout_flag(cabi) == 0
+
+
+@pytest.mark.parametrize("shape", [(5, 3), (257, 1023), (2048, 2048), (3000, 1111)], ids=lambda s: f"{s[0]}x{s[1]}")
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
+def test_resident_pair(cabi, shape, in_dtype):
+    x = util.normal_with_outliers(shape, 77, in_dtype)
+    modes = (1, 2, 3) if in_dtype == torch.bfloat16 else (3,)
+    for mode in modes:
+        (o4, o5, amax, scales), (p4, p5, amax2, scales2) = _both_paths(cabi, x.cuda(), lambda t: cabi.dynamic_scaled_quant_pair(t, mode))
+        r4, ramax, rs4 = co.dynamic_scaled_quant(x, E4, getattr(co, MODE[mode]))
+        r5, _, rs5 = co.dynamic_scaled_quant(x, E5, getattr(co, MODE[mode]))
+        assert torch.equal(util.codes(o4), r4) and torch.equal(util.codes(o5), r5)
+        assert torch.equal(util.codes(p4), r4) and torch.equal(util.codes(p5), r5)
+        assert amax.item() == ramax.item() and scales.tolist() == [rs4.item(), rs5.item()] == scales2.tolist()
+        # the identity the shared product relies on
+        assert scales[1].item() == 128.0 * scales[0].item()
+
+
+@pytest.mark.parametrize("amax", [1e-30, 3e-13, 1e-12, 7.3e-5, 0.1, 1.0, 3.14159, 448.0, 57344.0, 6.5e4, 1e20, 3.3e38])
+def test_e5m2_scale_is_128_times_e4m3_scale(amax):
+    """the pair kernel derives the e5m2 operand from the e4m3 one: fmax ratio 57344 / 448 = 2^7"""
+    assert co.amax_to_scale(amax, E5) == 128.0 * co.amax_to_scale(amax, E4)
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
+def test_resident_special_values(cabi, in_dtype):
+    """an infinity makes the scale 0 and inf * 0 a NaN; a NaN makes everything NaN: both take the
+    kernel's re-read path and must equal the two-kernel result and the oracle"""
+    for special in (float("inf"), float("-inf"), float("nan")):
+        x = util.normal((300, 257), 5, in_dtype)
+        x[17, 3] = special
+        # (a NaN times a NaN scale keeps the sign of whichever operand the multiplier picks: use one sign)
+        x[299, 256] = special if special != special else -special
+        (o4, o5, amax, _), (p4, p5, amax2, _) = _both_paths(cabi, x.cuda(), lambda t: cabi.dynamic_scaled_quant_pair(t, 2 if in_dtype == torch.bfloat16 else 3))
+        r4, ramax, _ = co.dynamic_scaled_quant(x, E4, co.ROUND_V2 if in_dtype == torch.bfloat16 else co.ROUND_V3)
+        assert torch.equal(util.codes(o4), r4) and torch.equal(util.codes(p4), r4)
+        assert torch.equal(util.codes(o5), util.codes(p5))
+        assert (amax.item() == ramax.item()) or (amax.item() != amax.item() and ramax.item() != ramax.item())
+    x = torch.zeros((64, 64), dtype=in_dtype)
+    o4, o5, amax, scales = cabi.dynamic_scaled_quant_pair(x.cuda(), 3)
+    assert amax.item() == 0.0 and not util.codes(o4).any() and not util.codes(o5).any()
+    assert _timeout_flag(cabi) == 0
+
+
+def test_resident_capacity_boundary(cabi):
+    """8192 x 8192 bf16 (and 8192 x 4096 fp32) is exactly what 256 CUs hold; one more row does not
+    fit and goes through the two kernels"""
+    cabi.set_tuning("dynamic.resident", 1)
+    for shape, dtype in (((8192, 8192), torch.bfloat16), ((8192, 4096), torch.float32), ((8193, 8192), torch.bfloat16)):
+        x = util.normal_with_outliers(shape, 1002, dtype)
+        o4, o5, amax, scales = cabi.dynamic_scaled_quant_pair(x.cuda(), 2 if dtype == torch.bfloat16 else 3)
+        mode = co.ROUND_V2 if dtype == torch.bfloat16 else co.ROUND_V3
+        r4, ramax, rs4 = co.dynamic_scaled_quant(x, E4, mode)
+        r5, _, rs5 = co.dynamic_scaled_quant(x, E5, mode)
+        assert torch.equal(util.codes(o4), r4) and torch.equal(util.codes(o5), r5)
+        assert amax.item() == ramax.item() and scales.tolist() == [rs4.item(), rs5.item()]
+    assert _timeout_flag(cabi) == 0
+
+
+def test_resident_back_to_back_and_two_streams(cabi):
+    """the workspace re-arms itself between launches of different sizes, and launches from two
+    streams are chained by the host instead of sharing the chip"""
+    cabi.set_tuning("dynamic.resident", 1)
+    xs = [util.normal_with_outliers(s, 9 + i) for i, s in enumerate([(2048, 2048), (100, 37), (4096, 1024), (64, 64)])]
+    refs = [co.dynamic_scaled_quant(x, E4, co.ROUND_V2)[0] for x in xs]
+    gx = [x.cuda() for x in xs]
+    outs = [cabi.dynamic_scaled_quant(g, E4, 2)[0] for g in gx for _ in range(2)]
+    for i, o in enumerate(outs):
+        assert torch.equal(util.codes(o), refs[i // 2])
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    results = []
+    for rep in range(6):
+        st = streams[rep % 2]
+        with torch.cuda.stream(st):
+            results.append((rep % len(xs), cabi.dynamic_scaled_quant(gx[rep % len(xs)], E4, 2)[0]))
+    torch.cuda.synchronize()
+    for i, o in results:
+        assert torch.equal(util.codes(o), refs[i])
+    for st in streams:
+        with torch.cuda.stream(st):
+            ws = cabi.workspace(torch.device("cuda"))
+            torch.cuda.synchronize()
+            assert int(ws[196:200].cpu().view(torch.int32).item()) == 0
+
+
+def test_resident_wait_gives_up_loudly(cabi):
+    """with a spin limit of one poll most workgroups stop waiting before the last one has arrived:
+    every wave still runs to the end, the sticky flag is set and those workgroups write NaN"""
+    cabi.set_tuning("dynamic.resident", 1)
+    cabi.set_tuning("dynamic.resident_spin_limit", 1)
+    x = util.normal((8192, 2048), 3).cuda()
+    out, amax, scale = cabi.dynamic_scaled_quant(x, E4, 2)
+    torch.cuda.synchronize()
+    assert _timeout_flag(cabi) == 1
+    codes = util.codes(out)
+    assert ((codes & 0x7F) == 0x7F).any()
+    # re-initialise the workspace (clears the flag) and check that the next call is right again
+    cabi.set_tuning("dynamic.resident_spin_limit", 1 << 19)
+    ws = cabi.workspace(torch.device("cuda"))
+    assert cabi.lib().dt_workspace_init(ws.data_ptr(), ws.numel(), None) == 0
+    torch.cuda.synchronize()
+    out, amax, scale = cabi.dynamic_scaled_quant(x, E4, 2)
+    ref, ramax, _ = co.dynamic_scaled_quant(x.cpu(), E4, co.ROUND_V2)
+    assert torch.equal(util.codes(out), ref) and amax.item() == ramax.item()
+    assert _timeout_flag(cabi) == 0
