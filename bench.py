@@ -241,6 +241,10 @@ def extra_kernels(torch, cabi, util, dev, K, W, gemm_only=False):
         hbm_row("saturated_cast", "fp32 [8192,8192] -> e4m3fn", n * 5,
                 lambda i: (rnd((8192, 8192), f32, i), torch.empty((8192, 8192), dtype=e4, device=dev)),
                 lambda x, o: cabi.saturated_cast(x, scale1, e4, cabi.ROUND_F32, o))
+        hbm_row("dynamic_scaled_quant (one resident kernel)", "bf16 [8192,8192] -> amax, scale, e4m3fn", n * 5,
+                lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
+                           torch.empty(1, device=dev), torch.empty(1, device=dev)),
+                lambda x, o, a, s_: cabi.dynamic_scaled_quant(x, e4, cabi.ROUND_BF16_SCALE_PRODUCT, o, a, s_))
         nr = 16384 * 4096
         for dt_, nm, b in ((f32, "fp32", 4), (bf16, "bf16", 2)):
             hbm_row("dynamic_scaled_quant_rowwise", f"config 3: {nm} [16384,4096] -> e4m3fn", nr * (b + 1) + 16384 * 8,
