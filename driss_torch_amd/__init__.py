@@ -4,7 +4,7 @@ The wrapper names, signatures and defaults follow the reference's
 ``driss_torch/__init__.py:20-122``; the work is done by hand-written gfx950 kernels in
 ``lib/libdriss_torch_hip.so`` (C ABI: ``include/driss_torch_hip.h``) reached through the
 registration shim ``lib/libdriss_torch.so``.  There is no fallback path: importing this
-package fails if the libraries have not been built (``python -m driss_torch_amd._build``).
+package fails if the libraries have not been built (``python driss_torch_amd/_build.py``).
 """
 from pathlib import Path
 from typing import Optional, Tuple
@@ -16,7 +16,7 @@ hip_lib_path = _LIB_DIR / "libdriss_torch_hip.so"
 lib_path = _LIB_DIR / "libdriss_torch.so"
 for _p in (hip_lib_path, lib_path):
     if not _p.exists():
-        raise ImportError(f"{_p} is missing: build it with `python -m driss_torch_amd._build`")
+        raise ImportError(f"{_p} is missing: build it with `python driss_torch_amd/_build.py`")
 torch.ops.load_library(str(lib_path.resolve()))
 torch.ops.import_module("driss_torch_amd.abstract_impls")
 
@@ -114,6 +114,15 @@ def mx_fp8_quantize_blocked(input: Tensor, axis: int = 1, ScalarType: torch.dtyp
     """MXFP8 cast whose scales come out in the blocked layout ``mx_fp8_bf16`` reads, with K as
     the contiguous payload dimension: axis 1 -> payload [M, N]; axis 0 -> payload [N, M]."""
     return ops.mx_fp8_quantize_ex(input, 32, axis, axis % 2 == 0, ScalarType, True)
+
+
+def mx_fp8_quantize_dual(input: Tensor, ScalarType: torch.dtype = torch.float8_e4m3fn, blocked: bool = False
+                         ) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """Both MXFP8 blockings of ``input`` [M, N] from one read: ``(data [M, N], scale, data_t [N, M],
+    scale_t)``.  The first pair equals ``mx_fp8_quantize(input)``, the second
+    ``mx_fp8_quantize(input.t().contiguous())``: the operand for a forward product and the one for the
+    weight-gradient product.  ``blocked`` selects the scale layout ``mx_fp8_bf16`` reads."""
+    return ops.mx_fp8_quantize_dual(input, ScalarType, blocked)
 
 
 def to_blocked(scale: Tensor) -> Tensor:

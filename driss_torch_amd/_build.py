@@ -5,7 +5,7 @@
 * ``lib/libdriss_torch.so``     -- the ``torch.ops.DrissTorch`` registration shim, host C++
   only, linked against torch and the kernel library.
 
-Run ``python -m driss_torch_amd._build`` (or ``__graft_entry__.build()``).  The GPU is not
+Run ``python driss_torch_amd/_build.py`` (or ``__graft_entry__.build()``).  The GPU is not
 needed: hipcc cross-compiles.
 """
 from __future__ import annotations

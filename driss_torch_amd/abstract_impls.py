@@ -74,6 +74,15 @@ def mx_fp8_quantize_ex_meta(x, block_size, axis, transpose, fp8_type, blocked):
             torch.empty((scale_elems,), dtype=torch.float8_e8m0fnu, device=x.device))
 
 
+@register_fake("DrissTorch::mx_fp8_quantize_dual")
+def mx_fp8_quantize_dual_meta(x, fp8_type, blocked):
+    shape_r, scale_r = _mx_shapes(x, 1, False, blocked)
+    shape_c, scale_c = _mx_shapes(x, 0, True, blocked)
+    e8 = torch.float8_e8m0fnu
+    return (torch.empty(shape_r, dtype=fp8_type, device=x.device), torch.empty((scale_r,), dtype=e8, device=x.device),
+            torch.empty(shape_c, dtype=fp8_type, device=x.device), torch.empty((scale_c,), dtype=e8, device=x.device))
+
+
 @register_fake("DrissTorch::to_blocked")
 def to_blocked_meta(scale):
     r, c = scale.shape

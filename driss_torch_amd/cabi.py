@@ -37,6 +37,7 @@ SIGNATURES = {
     "dt_saturated_cast_pair": (_i32, [_vp, _i32, _i64, _vp, _i32, _vp, _vp, _vp]),
     "dt_dynamic_scaled_quant_rowwise": (_i32, [_vp, _i32, _i64, _i64, _i32, _vp, _vp, _vp, _vp]),
     "dt_mx_fp8_quantize": (_i32, [_vp, _i32, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
+    "dt_mx_fp8_quantize_dual": (_i32, [_vp, _i32, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "dt_blocked_scale_bytes": (_i64, [_i64, _i64]),
     "dt_to_blocked": (_i32, [_vp, _i64, _i64, _vp, _vp]),
     "dt_mx_fp8_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
@@ -53,7 +54,7 @@ def lib() -> C.CDLL:
     global _lib
     if _lib is None:
         if not _LIB_PATH.exists():
-            raise ImportError(f"{_LIB_PATH} is missing: build it with `python -m driss_torch_amd._build`")
+            raise ImportError(f"{_LIB_PATH} is missing: build it with `python driss_torch_amd/_build.py`")
         L = C.CDLL(str(_LIB_PATH))
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(L, name)
@@ -197,6 +198,21 @@ def mx_fp8_quantize(x: torch.Tensor, axis: int = 1, transpose: bool = False, out
     _check(lib().dt_mx_fp8_quantize(x.data_ptr(), IN_DTYPE[x.dtype], R, Cc, axis, int(transpose), OUT_DTYPE[out_dtype],
                                     layout, data.data_ptr(), scale.data_ptr(), _stream()), "dt_mx_fp8_quantize")
     return data, scale
+
+
+def mx_fp8_quantize_dual(x: torch.Tensor, out_dtype: torch.dtype = torch.float8_e4m3fn, layout: int = SCALE_PLAIN):
+    """(data_rows, scale_rows, data_cols_t, scale_cols_t): the (axis 1) cast of x and the (axis 1) cast of x^T
+    from one read of x."""
+    R, Cc = x.shape
+    dr_shape, sr_shape = mx_shapes(R, Cc, 1, False, layout)
+    dc_shape, sc_shape = mx_shapes(R, Cc, 0, True, layout)
+    dr = torch.empty(dr_shape, dtype=out_dtype, device=x.device)
+    sr = torch.empty(sr_shape, dtype=torch.uint8, device=x.device)
+    dc = torch.empty(dc_shape, dtype=out_dtype, device=x.device)
+    sc = torch.empty(sc_shape, dtype=torch.uint8, device=x.device)
+    _check(lib().dt_mx_fp8_quantize_dual(x.data_ptr(), IN_DTYPE[x.dtype], R, Cc, OUT_DTYPE[out_dtype], layout, dr.data_ptr(),
+                                         sr.data_ptr(), dc.data_ptr(), sc.data_ptr(), _stream()), "dt_mx_fp8_quantize_dual")
+    return dr, sr, dc, sc
 
 
 def to_blocked(scale: torch.Tensor) -> torch.Tensor:

@@ -25,6 +25,8 @@ Knob g_knobs[] = {
     {"cast.pair_blocks_per_cu", 3},
     {"mx.blocks_per_cu", 16},
     {"mx.col_blocks_per_cu", 16},
+    {"mx.dual", 1},
+    {"mx.row_band4", 1},
     {"gemm.variant", 0},
     {"dynamic.resident", 1},
     {"dynamic.resident_min_kib", 1024},

@@ -24,6 +24,13 @@ int launch_mx(const MxArgs& a) {
     int64_t waves = (int64_t)cus * tuning("mx.blocks_per_cu") * (kBlock / kWave);
     if (waves > nsuper) waves = nsuper;
     const unsigned grid = (unsigned)ceil_div(waves, kBlock / kWave);
+    if constexpr (LAYOUT == DT_SCALE_BLOCKED) {
+      if (a.rows % 128 == 0 && a.cols % 512 == 0 && tuning("mx.row_band4")) {
+        mx_row_kernel<IN, OUT, LAYOUT, true><<<grid, kBlock, 0, a.stream>>>(a.x, (uint32_t)nblocks, (uint32_t)(a.cols / 32),
+                                                                           a.data, a.scale);
+        return launch_status();
+      }
+    }
     mx_row_kernel<IN, OUT, LAYOUT><<<grid, kBlock, 0, a.stream>>>(a.x, (uint32_t)nblocks, (uint32_t)(a.cols / 32),
                                                                  a.data, a.scale);
     return launch_status();
@@ -73,6 +80,41 @@ int launch_mx_in(const MxArgs& a, int out_dtype, int layout) {
     return layout == DT_SCALE_BLOCKED ? launch_mx<IN, DT_E4M3FN, DT_SCALE_BLOCKED>(a) : launch_mx<IN, DT_E4M3FN, DT_SCALE_PLAIN>(a);
   return layout == DT_SCALE_BLOCKED ? launch_mx<IN, DT_E5M2, DT_SCALE_BLOCKED>(a) : launch_mx<IN, DT_E5M2, DT_SCALE_PLAIN>(a);
 }
+
+struct DualArgs {
+  const void* x;
+  int64_t rows, cols;
+  uint8_t *data_r, *scale_r, *data_c, *scale_c;
+  hipStream_t stream;
+};
+
+// DT_OK when the one-read kernel was launched, kNotTaken when the shape or an alignment rules it out
+constexpr int kNotTaken = -1;
+template <int IN, int OUT, int LAYOUT>
+int launch_dual(const DualArgs& a) {
+  constexpr int kTileCols = 32 * InTraits<IN>::kVec;
+  if (!aligned(a.x, 16) || !aligned(a.data_r, 8) || !aligned(a.data_c, 16) || !aligned(a.scale_r, 4) ||
+      !aligned(a.scale_c, 4) || a.rows >= (1ll << 31) || a.cols >= (1ll << 31))
+    return kNotTaken;
+  const int64_t tiles = ceil_div(a.rows, (int64_t)kDualRows) * ceil_div(a.cols, (int64_t)kTileCols);
+  if (tiles > 0x7FFFFFFFll) return kNotTaken;
+  mx_dual_kernel<IN, OUT, LAYOUT><<<(unsigned)tiles, kBlock, 0, a.stream>>>(a.x, (uint32_t)a.rows, (uint32_t)a.cols, a.data_r,
+                                                                           a.scale_r, a.data_c, a.scale_c, a.cols <= a.rows ? 1 : 0);
+  return launch_status();
+}
+template <int IN>
+int launch_dual_in(const DualArgs& a, int out_dtype, int layout) {
+  if (out_dtype == DT_E4M3FN)
+    return layout == DT_SCALE_BLOCKED ? launch_dual<IN, DT_E4M3FN, DT_SCALE_BLOCKED>(a) : launch_dual<IN, DT_E4M3FN, DT_SCALE_PLAIN>(a);
+  return layout == DT_SCALE_BLOCKED ? launch_dual<IN, DT_E5M2, DT_SCALE_BLOCKED>(a) : launch_dual<IN, DT_E5M2, DT_SCALE_PLAIN>(a);
+}
+
+int zero_blocked_padding(uint8_t* scale, int64_t SR, int64_t SC, hipStream_t s) {
+  if (SR % 128 == 0 && SC % 4 == 0) return DT_OK;  // the cast writes every byte
+  const int64_t n = dt_blocked_scale_bytes(SR, SC);
+  dt::fill_bytes_kernel<<<(unsigned)std::min<int64_t>(dt::ceil_div(n, 256), 4096), 256, 0, s>>>(scale, n, 0);
+  return dt::launch_status();
+}
 }  // namespace
 
 extern "C" int64_t dt_blocked_scale_bytes(int64_t R, int64_t C) {
@@ -94,13 +136,8 @@ extern "C" int dt_mx_fp8_quantize(const void* x, int in_dtype, int64_t rows, int
   if (!x || !data || !scale) return DT_ERR_NULL_POINTER;
   if (!dt::aligned(x, in_dtype == DT_F32 ? 4 : 2)) return DT_ERR_MISALIGNED;
   hipStream_t s = dt::as_hip(stream);
-  if (scale_layout == DT_SCALE_BLOCKED) {
-    const int64_t SR = axis == 1 ? rows : cols, SC = (axis == 1 ? cols : rows) / 32;
-    if (SR % 128 != 0 || SC % 4 != 0) {  // zero the padding the cast itself never writes
-      const int64_t n = dt_blocked_scale_bytes(SR, SC);
-      dt::fill_bytes_kernel<<<(unsigned)std::min<int64_t>(dt::ceil_div(n, 256), 4096), 256, 0, s>>>(scale, n, 0);
-      if (int st = dt::launch_status()) return st;
-    }
+  if (scale_layout == DT_SCALE_BLOCKED) {  // zero the padding the cast itself never writes
+    if (int st = zero_blocked_padding(scale, axis == 1 ? rows : cols, (axis == 1 ? cols : rows) / 32, s)) return st;
   }
   MxArgs a{x, rows, cols, axis, transpose, static_cast<uint8_t*>(data), scale, s};
   switch (in_dtype) {
@@ -108,6 +145,37 @@ extern "C" int dt_mx_fp8_quantize(const void* x, int in_dtype, int64_t rows, int
     case DT_BF16: return launch_mx_in<DT_BF16>(a, out_dtype, scale_layout);
     default: return launch_mx_in<DT_F16>(a, out_dtype, scale_layout);
   }
+}
+
+extern "C" int dt_mx_fp8_quantize_dual(const void* x, int in_dtype, int64_t rows, int64_t cols, int out_dtype, int scale_layout,
+                                       void* data_rows, uint8_t* scale_rows, void* data_cols_t, uint8_t* scale_cols_t,
+                                       dt_stream_t stream) {
+  if (in_dtype != DT_F32 && in_dtype != DT_BF16 && in_dtype != DT_F16) return DT_ERR_INVALID_DTYPE;
+  if (out_dtype != DT_E4M3FN && out_dtype != DT_E5M2) return DT_ERR_INVALID_DTYPE;
+  if (scale_layout != DT_SCALE_PLAIN && scale_layout != DT_SCALE_BLOCKED) return DT_ERR_INVALID_MODE;
+  if (rows < 0 || cols < 0 || rows % 32 != 0 || cols % 32 != 0) return DT_ERR_INVALID_SHAPE;
+  if (rows == 0 || cols == 0) return DT_OK;
+  if (!x || !data_rows || !scale_rows || !data_cols_t || !scale_cols_t) return DT_ERR_NULL_POINTER;
+  if (!dt::aligned(x, in_dtype == DT_F32 ? 4 : 2)) return DT_ERR_MISALIGNED;
+  hipStream_t s = dt::as_hip(stream);
+  DualArgs a{x, rows, cols, static_cast<uint8_t*>(data_rows), scale_rows, static_cast<uint8_t*>(data_cols_t), scale_cols_t, s};
+  const bool fast_ok = dt::tuning("mx.dual") != 0;
+  if (fast_ok) {
+    if (scale_layout == DT_SCALE_BLOCKED) {
+      if (int st = zero_blocked_padding(scale_rows, rows, cols / 32, s)) return st;
+      if (int st = zero_blocked_padding(scale_cols_t, cols, rows / 32, s)) return st;
+    }
+    int st;
+    switch (in_dtype) {
+      case DT_F32: st = launch_dual_in<DT_F32>(a, out_dtype, scale_layout); break;
+      case DT_BF16: st = launch_dual_in<DT_BF16>(a, out_dtype, scale_layout); break;
+      default: st = launch_dual_in<DT_F16>(a, out_dtype, scale_layout); break;
+    }
+    if (st != kNotTaken) return st;
+  }
+  // two passes over x
+  if (int st = dt_mx_fp8_quantize(x, in_dtype, rows, cols, 1, 0, out_dtype, scale_layout, data_rows, scale_rows, stream)) return st;
+  return dt_mx_fp8_quantize(x, in_dtype, rows, cols, 0, 1, out_dtype, scale_layout, data_cols_t, scale_cols_t, stream);
 }
 
 extern "C" int dt_to_blocked(const uint8_t* scale, int64_t R, int64_t C, uint8_t* out, dt_stream_t stream) {

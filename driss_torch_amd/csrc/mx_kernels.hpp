@@ -8,6 +8,8 @@
 //                  a 32-row tile and merge their column maxima through LDS.
 //  mx_col_t_kernel blocks down columns, payload transposed through LDS so that the stores
 //                  are full 128-byte rows of the [cols, rows] output.
+//  mx_dual_kernel  blocks along rows (payload as is) and down columns (payload transposed) from
+//                  one read of the input.
 //  mx_any_kernel   one thread per block, arbitrary strides: covers every (axis, transpose)
 //                  pair and shapes the fast kernels do not take.
 #pragma once
@@ -38,7 +40,8 @@ __device__ __forceinline__ int64_t scale_offset(int64_t r, int64_t c, int64_t C)
 template <int OUT>
 struct MxScale {
   uint32_t byte;  // 0..254, or 255 for a block that holds a NaN
-  float mult;
+  float mult;     // 2^(127-b): what the block is multiplied by
+  float scale;    // 2^(b-127) as the scaled conversion instructions take it (they divide by it)
   bool nan;
 };
 template <int OUT>
@@ -54,6 +57,7 @@ __device__ __forceinline__ MxScale<OUT> mx_scale_from_absbits(uint32_t absbits) 
   r.nan = absbits > 0x7F800000u;
   r.byte = r.nan ? 255u : (uint32_t)b;
   r.mult = as_f32((uint32_t)(254 - b) << 23);       // b <= 248 for any input, so never 2^-127
+  r.scale = as_f32((uint32_t)b << 23);              // only the exponent field is read: 0 stands for 2^-127
   return r;
 }
 
@@ -62,6 +66,75 @@ template <int OUT>
 __device__ __forceinline__ uint32_t pack4_finite(float p0, float p1, float p2, float p3) {
   uint32_t w = cvt_pk<OUT, false>(clamp_fp8<OUT>(p0), clamp_fp8<OUT>(p1), 0u);
   return cvt_pk<OUT, true>(clamp_fp8<OUT>(p2), clamp_fp8<OUT>(p3), w);
+}
+
+// ---- conversions that apply the block scale themselves (v_cvt_scalef32_pk_{fp8,bf8}_{bf16,f16,f32})
+// One instruction turns two inputs into two fp8 bytes of x / 2^(b-127), rounded to nearest even.
+// With MODE.FP16_OVFL set they saturate (infinity included) instead of producing NaN / infinity,
+// which makes them bit-identical to multiply, clamp, convert for every non-NaN input and every
+// scale byte 0..248 (checked exhaustively over all bf16 and f16 patterns and 9 x 65536 fp32
+// patterns per byte on the hardware).  A NaN input gives a NaN code other than 0x7F, so blocks
+// that hold a NaN are still overwritten wholesale by the callers.
+typedef short v2s16 __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf16 __attribute__((ext_vector_type(2)));
+typedef _Float16 v2f16 __attribute__((ext_vector_type(2)));
+
+// every wave of a kernel that uses them calls this first (the mode register is per wave)
+__device__ __forceinline__ void saturate_fp8_conversions() { __builtin_amdgcn_s_setreg(1 | (23 << 6), 1); }
+
+// two 16-bit inputs packed in one word -> bytes 0-1 (HI false) or 2-3 (HI true) of old
+template <int IN, int OUT, bool HI>
+__device__ __forceinline__ uint32_t cvt_scaled_pair16(uint32_t old, uint32_t pair, float scale) {
+  static_assert(IN == DT_BF16 || IN == DT_F16, "16-bit inputs");
+  const v2s16 o = __builtin_bit_cast(v2s16, old);
+  v2s16 r;
+  if constexpr (IN == DT_BF16) {
+    const v2bf16 x = __builtin_bit_cast(v2bf16, pair);
+    if constexpr (OUT == DT_E5M2) r = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(o, x, scale, HI);
+    else r = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o, x, scale, HI);
+  } else {
+    const v2f16 x = __builtin_bit_cast(v2f16, pair);
+    if constexpr (OUT == DT_E5M2) r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f16(o, x, scale, HI);
+    else r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(o, x, scale, HI);
+  }
+  return __builtin_bit_cast(uint32_t, r);
+}
+template <int OUT, bool HI>
+__device__ __forceinline__ uint32_t cvt_scaled_pair32(uint32_t old, uint32_t a, uint32_t b, float scale) {
+  const v2s16 o = __builtin_bit_cast(v2s16, old);
+  v2s16 r;
+  if constexpr (OUT == DT_E5M2) r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(o, as_f32(a), as_f32(b), scale, HI);
+  else r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(o, as_f32(a), as_f32(b), scale, HI);
+  return __builtin_bit_cast(uint32_t, r);
+}
+// four 16-bit inputs in two words, or four fp32 words -> one word of fp8, all with one scale
+template <int IN, int OUT>
+__device__ __forceinline__ uint32_t cvt_scaled_4x16(uint32_t w0, uint32_t w1, float scale) {
+  return cvt_scaled_pair16<IN, OUT, true>(cvt_scaled_pair16<IN, OUT, false>(w0, w0, scale), w1, scale);
+}
+template <int OUT>
+__device__ __forceinline__ uint32_t cvt_scaled_4x32(uint32_t a, uint32_t b, uint32_t c, uint32_t d, float scale) {
+  return cvt_scaled_pair32<OUT, true>(cvt_scaled_pair32<OUT, false>(a, a, b, scale), c, d, scale);
+}
+// low (half 0) or high (half 1) 16 bits of a and of b as one word {a.half, b.half}
+__device__ __forceinline__ uint32_t gather_halves(int half, uint32_t a, uint32_t b) {
+  return __builtin_amdgcn_perm(b, a, half ? 0x07060302u : 0x05040100u);
+}
+// Four adjacent elements with four different scales (blocks down the columns, payload in place).
+// A conversion writes two bytes with one scale; the byte that belongs to the other scale is
+// overwritten or dropped by the byte permute at the end.
+template <int IN, int OUT>
+__device__ __forceinline__ uint32_t cvt_scaled_4x16_each(uint32_t w0, uint32_t w1, const float* sc /* 4 scales */) {
+  // byte 0 = w.lo / sc[0], byte 3 = w.hi / sc[1]
+  const uint32_t u0 = cvt_scaled_pair16<IN, OUT, true>(cvt_scaled_pair16<IN, OUT, false>(w0, w0, sc[0]), w0, sc[1]);
+  const uint32_t u1 = cvt_scaled_pair16<IN, OUT, true>(cvt_scaled_pair16<IN, OUT, false>(w1, w1, sc[2]), w1, sc[3]);
+  return __builtin_amdgcn_perm(u1, u0, 0x07040300u);
+}
+template <int OUT>
+__device__ __forceinline__ uint32_t cvt_scaled_4x32_each(uint32_t a, uint32_t b, uint32_t c, uint32_t d, const float* sc) {
+  const uint32_t e = cvt_scaled_pair32<OUT, true>(cvt_scaled_pair32<OUT, false>(a, a, a, sc[0]), c, c, sc[2]);  // bytes 0, 2
+  const uint32_t o = cvt_scaled_pair32<OUT, true>(cvt_scaled_pair32<OUT, false>(b, b, b, sc[1]), d, d, sc[3]);  // bytes 1, 3
+  return __builtin_amdgcn_perm(o, e, 0x07020500u);
 }
 
 template <int IN>
@@ -105,10 +178,17 @@ __device__ __forceinline__ uint32_t vec_absmax_bits(u32x4 w) {
 // The matrix is a flat run of 32-element blocks.  One wave pass ("super-chunk") covers 64
 // blocks as LPB chunks of 64 vectors; lane l ends up holding the scale byte of chunk
 // l % LPB, block l / LPB, so the 64 scale bytes leave in a single store instruction.
-template <int IN, int OUT, int LAYOUT>
+//
+// BAND4 (blocked scale layout, rows % 128 == 0, cols % 512 == 0): a pass covers 4 rows x 512
+// elements instead -- rows q, q+32, q+64, q+96 of a 128-row band, one chunk (fp32: two) per
+// row -- because those are the scales that sit next to each other in the blocked layout: the 64
+// bytes of a pass then fall into 4 runs of 16 bytes instead of 16 runs of 4, which costs a
+// quarter of the memory transactions (36.8 -> 33 us at 8192 x 8192 bf16).
+template <int IN, int OUT, int LAYOUT, bool BAND4 = false>
 __global__ __launch_bounds__(kBlock) void mx_row_kernel(const void* __restrict__ x, uint32_t nblocks,
                                                         uint32_t kblocks, uint8_t* __restrict__ data,
                                                         uint8_t* __restrict__ scale) {
+  static_assert(!BAND4 || LAYOUT == DT_SCALE_BLOCKED, "the 4-row pass exists for the blocked layout");
   constexpr int kV = InTraits<IN>::kVec;      // elements per vector
   constexpr int LPB = 32 / kV;                // lanes per block: 4 or 8
   constexpr int BPC = kWave / LPB;            // blocks per chunk: 16 or 8
@@ -118,38 +198,53 @@ __global__ __launch_bounds__(kBlock) void mx_row_kernel(const void* __restrict__
   const uint32_t nsuper = (nblocks + 63u) / 64u;
   const uint32_t wave_id = (blockIdx.x * kBlock + threadIdx.x) / kWave;
   const uint32_t nwaves = gridDim.x * (kBlock / kWave);
+  saturate_fp8_conversions();
 
+  const uint32_t segs = kblocks / 16u;                 // BAND4: 512-element segments per row
+  const uint32_t row_vecs = kblocks * (uint32_t)LPB;   // vectors per row
   for (uint32_t sc = wave_id; sc < nsuper; sc += nwaves) {
-    const uint32_t vbase = sc * 64u * LPB + lane;
+    // vector index of chunk c of this pass
+    uint32_t band_row = 0, seg = 0;
+    if constexpr (BAND4) {
+      const uint32_t band = sc / (32u * segs), rem = sc - band * 32u * segs, q = rem / segs;
+      seg = rem - q * segs;
+      band_row = band * 128u + q;
+    }
+    auto vec_index = [&](int c) -> uint32_t {
+      if constexpr (BAND4) return (band_row + 32u * (c & 3)) * row_vecs + seg * (16u * LPB) + (uint32_t)(c >> 2) * kWave + lane;
+      else return sc * 64u * LPB + c * kWave + lane;
+    };
     u32x4 w[LPB];
 #pragma unroll
     for (int c = 0; c < LPB; ++c) {
-      const uint32_t vi = vbase + c * kWave;
+      const uint32_t vi = vec_index(c);
       w[c] = vi < nvec ? ld_stream(v + vi) : u32x4{0u, 0u, 0u, 0u};
     }
     uint32_t mybyte = 0;
 #pragma unroll
     for (int c = 0; c < LPB; ++c) {
-      const uint32_t vi = vbase + c * kWave;
+      const uint32_t vi = vec_index(c);
       uint32_t m = quad_umax(vec_absmax_bits<IN>(w[c]));
       if constexpr (LPB == 8) m = umax(m, dpp<kDppRowHalfMirror>(m));
       const MxScale<OUT> s = mx_scale_from_absbits<OUT>(m);
       if ((lane % LPB) == c) mybyte = s.byte;
       if (vi < nvec) {
         if constexpr (IN == DT_F32) {
-          uint32_t r = pack4_finite<OUT>(as_f32(w[c].x) * s.mult, as_f32(w[c].y) * s.mult, as_f32(w[c].z) * s.mult,
-                                         as_f32(w[c].w) * s.mult);
+          const uint32_t r = cvt_scaled_4x32<OUT>(w[c].x, w[c].y, w[c].z, w[c].w, s.scale);
           st_stream(reinterpret_cast<uint32_t*>(data) + vi, s.nan ? 0x7F7F7F7Fu : r);
         } else {
-          float f[8];
-          unpack8<IN>(w[c], f);
           u32x2 r;
-          r.x = pack4_finite<OUT>(f[0] * s.mult, f[1] * s.mult, f[2] * s.mult, f[3] * s.mult);
-          r.y = pack4_finite<OUT>(f[4] * s.mult, f[5] * s.mult, f[6] * s.mult, f[7] * s.mult);
+          r.x = cvt_scaled_4x16<IN, OUT>(w[c].x, w[c].y, s.scale);
+          r.y = cvt_scaled_4x16<IN, OUT>(w[c].z, w[c].w, s.scale);
           if (s.nan) r = u32x2{0x7F7F7F7Fu, 0x7F7F7F7Fu};
           st_stream(reinterpret_cast<u32x2*>(data) + vi, r);
         }
       }
+    }
+    if constexpr (BAND4) {
+      const uint32_t c = lane % LPB, b = lane / LPB;   // mybyte: chunk c, block b of that chunk
+      scale[blocked_offset(band_row + 32u * (c & 3), seg * 16u + (c >> 2) * BPC + b, kblocks >> 2)] = (uint8_t)mybyte;
+      continue;
     }
     const uint32_t g = sc * 64u + (lane % LPB) * BPC + lane / LPB;  // block index of mybyte
     if (g < nblocks) {
@@ -237,13 +332,13 @@ __global__ __launch_bounds__(kBlock) void mx_col_kernel(const void* __restrict__
       cm[0] = as_u32(f16_lo(pm.x)); cm[1] = as_u32(f16_hi(pm.x)); cm[2] = as_u32(f16_lo(pm.y)); cm[3] = as_u32(f16_hi(pm.y));
       cm[4] = as_u32(f16_lo(pm.z)); cm[5] = as_u32(f16_hi(pm.z)); cm[6] = as_u32(f16_lo(pm.w)); cm[7] = as_u32(f16_hi(pm.w));
     }
-    float mult[kV];
+    float scl[kV];
     uint32_t nanmask[kW] = {};
     uint32_t bytes[kW] = {};  // the kV scale bytes packed in column order
 #pragma unroll
     for (int c = 0; c < kV; ++c) {
       const MxScale<OUT> sc = mx_scale_from_absbits<OUT>(cm[c]);
-      mult[c] = sc.mult;
+      scl[c] = sc.scale;
       bytes[c / 4] |= sc.byte << (8 * (c % 4));
       nanmask[c / 4] |= sc.nan ? (0xFFu << (8 * (c % 4))) : 0u;
     }
@@ -251,19 +346,15 @@ __global__ __launch_bounds__(kBlock) void mx_col_kernel(const void* __restrict__
       uint8_t* drow = data + (uint64_t)(tr * 32u + w * 8u) * cols + col0;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        float f[8];
-        if constexpr (IN == DT_F32) {
-          f[0] = as_f32(v[i].x); f[1] = as_f32(v[i].y); f[2] = as_f32(v[i].z); f[3] = as_f32(v[i].w);
-        } else {
-          unpack8<IN>(v[i], f);
-        }
         uint32_t r[kW];
-#pragma unroll
-        for (int q = 0; q < kW; ++q) {
-          r[q] = pack4_finite<OUT>(f[4 * q] * mult[4 * q], f[4 * q + 1] * mult[4 * q + 1], f[4 * q + 2] * mult[4 * q + 2],
-                                   f[4 * q + 3] * mult[4 * q + 3]);
-          r[q] = (r[q] & ~nanmask[q]) | (0x7F7F7F7Fu & nanmask[q]);
+        if constexpr (IN == DT_F32) {
+          r[0] = cvt_scaled_4x32_each<OUT>(v[i].x, v[i].y, v[i].z, v[i].w, scl);
+        } else {
+          r[0] = cvt_scaled_4x16_each<IN, OUT>(v[i].x, v[i].y, scl);
+          r[1] = cvt_scaled_4x16_each<IN, OUT>(v[i].z, v[i].w, scl + 4);
         }
+#pragma unroll
+        for (int q = 0; q < kW; ++q) r[q] = (r[q] & ~nanmask[q]) | (0x7F7F7F7Fu & nanmask[q]);
         if constexpr (kW == 2) st_stream(reinterpret_cast<u32x2*>(drow + (uint64_t)i * cols), u32x2{r[0], r[1]});
         else st_stream(reinterpret_cast<uint32_t*>(drow + (uint64_t)i * cols), r[0]);
       }
@@ -277,6 +368,7 @@ __global__ __launch_bounds__(kBlock) void mx_col_kernel(const void* __restrict__
 
   // part[] alternates between iterations, so one barrier per tile is enough: a wave can be at
   // most one barrier ahead of the slowest reader of the buffer it will write two tiles on
+  saturate_fp8_conversions();
   const uint32_t stride = gridDim.x;
   uint32_t t = blockIdx.x;  // < ntiles
   u32x4 va[8], vb[8];
@@ -323,6 +415,7 @@ __global__ __launch_bounds__(kBlock) void mx_col_t_kernel(const void* __restrict
   const uint32_t row0 = tr * kColTRows + w * 32, col0 = tc * kColTCols + lane * 4;
   const bool active = row0 < rows && col0 < cols;  // rows % 32 == 0 and cols % 4 == 0
 
+  saturate_fp8_conversions();
   uint32_t sbyte[4] = {0, 0, 0, 0};
   if (active) {
     // 32 rows x 4 columns kept packed as loaded: fp32 -> one 16-byte load per row, 16-bit -> one
@@ -333,14 +426,15 @@ __global__ __launch_bounds__(kBlock) void mx_col_t_kernel(const void* __restrict
     const uint8_t* p = static_cast<const uint8_t*>(x) + ((uint64_t)row0 * cols + col0) * kB;
 #pragma unroll
     for (int i = 0; i < 32; ++i) wv[i] = ld_stream(reinterpret_cast<const row_t*>(p + (uint64_t)i * cols * kB));
-    auto elem = [&](int i, int c) -> float {
-      if constexpr (IN == DT_F32) {
-        return as_f32(c == 0 ? wv[i].x : c == 1 ? wv[i].y : c == 2 ? wv[i].z : wv[i].w);
-      } else {
-        const uint32_t d = c < 2 ? wv[i].x : wv[i].y;
-        if constexpr (IN == DT_BF16) return (c & 1) ? bf16_hi(d) : bf16_lo(d);
-        else return (c & 1) ? f16_hi(d) : f16_lo(d);
-      }
+    // the word that holds column c of row i (fp32: the element itself; 16-bit: it and its neighbour)
+    auto word = [&](int i, int c) -> uint32_t {
+      if constexpr (IN == DT_F32) return c == 0 ? wv[i].x : c == 1 ? wv[i].y : c == 2 ? wv[i].z : wv[i].w;
+      else return c < 2 ? wv[i].x : wv[i].y;
+    };
+    auto elem = [&](int i, int c) -> float {  // (only for the column maxima of f16 / fp32 inputs)
+      if constexpr (IN == DT_F32) return as_f32(word(i, c));
+      else if constexpr (IN == DT_BF16) return (c & 1) ? bf16_hi(word(i, c)) : bf16_lo(word(i, c));
+      else return (c & 1) ? f16_hi(word(i, c)) : f16_lo(word(i, c));
     };
     if constexpr (IN == DT_BF16) {
       uint32_t p0 = 0, p1 = 0;
@@ -360,8 +454,11 @@ __global__ __launch_bounds__(kBlock) void mx_col_t_kernel(const void* __restrict
       uint32_t r[8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) {
-        r[q] = pack4_finite<OUT>(elem(4 * q, c) * s.mult, elem(4 * q + 1, c) * s.mult, elem(4 * q + 2, c) * s.mult,
-                                 elem(4 * q + 3, c) * s.mult);
+        if constexpr (IN == DT_F32)
+          r[q] = cvt_scaled_4x32<OUT>(word(4 * q, c), word(4 * q + 1, c), word(4 * q + 2, c), word(4 * q + 3, c), s.scale);
+        else
+          r[q] = cvt_scaled_4x16<IN, OUT>(gather_halves(c & 1, word(4 * q, c), word(4 * q + 1, c)),
+                                          gather_halves(c & 1, word(4 * q + 2, c), word(4 * q + 3, c)), s.scale);
         if (s.nan) r[q] = 0x7F7F7F7Fu;
       }
       u32x4* t = reinterpret_cast<u32x4*>(tile + (lane * 4 + c) * kColTPitch + w * 32);
@@ -396,6 +493,204 @@ __global__ __launch_bounds__(kBlock) void mx_col_t_kernel(const void* __restrict
 #pragma unroll
       for (int k = 0; k < 4; ++k)
         if (rb0 + k < RB) scale[scale_offset<LAYOUT>(c, rb0 + k, RB)] = (uint8_t)(sw >> (8 * k));
+    }
+  }
+}
+
+// -------------------------------- both blockings from one read of the input ("dual")
+// Row-wise cast in the input orientation plus the column-wise cast with a transposed payload:
+// the two operands a training step needs of one tensor (x for the forward product, x^T for the
+// weight gradient), from a single pass over x.  A workgroup owns 128 rows x 32*kV columns.  Wave
+// w takes rows 32w..32w+31: its lower 32 lanes hold rows 0..15 of those, the upper 32 lanes rows
+// 16..31, each lane kV adjacent columns (sixteen 16-byte loads; one load instruction of a wave
+// reads two contiguous row segments).  The row-block maximum is a max over the 4 (fp32: 8)
+// neighbouring lanes, the column-block maximum a lane-local max over 16 rows merged with the
+// other half of the wave.  Row payload and nothing else goes straight to memory; the column
+// payload is transposed through LDS as in mx_col_t_kernel, and both sets of scale bytes are
+// staged in LDS so that they leave as whole words.
+//
+// LDS tile: [column][128 rows] with a pitch of 144 bytes; the 16-byte chunk index is XORed
+// with bits 4..6 of the column so that the 16 lanes of one write phase (columns kV apart) fall
+// on 16 different bank groups.
+constexpr int kDualRows = 128, kDualPitch = 144;
+
+__device__ __forceinline__ uint32_t other_half_max_u32(uint32_t v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);  // [0]: lower half's value, [1]: upper half's
+  return umax(r[0], r[1]);
+}
+__device__ __forceinline__ uint32_t other_half_max_pk16(uint32_t v) {  // v: two 16-bit magnitudes
+  const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return pk_absmax16(r[0], r[1]);
+}
+
+template <int IN, int OUT, int LAYOUT>
+__global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict__ x, uint32_t rows, uint32_t cols,
+                                                         uint8_t* __restrict__ data_r, uint8_t* __restrict__ scale_r,
+                                                         uint8_t* __restrict__ data_c, uint8_t* __restrict__ scale_c, int cols_first) {
+  constexpr int kV = InTraits<IN>::kVec;     // columns per lane: 8 or 4
+  constexpr int kW = kV / 4;                 // fp8 words per lane and row
+  constexpr int kB = InTraits<IN>::kBytes;
+  constexpr int kTileCols = 32 * kV;         // 256 or 128
+  constexpr int kRowBlocks = kTileCols / 32; // row-direction blocks per tile row: 8 or 4
+  constexpr int LPB = 32 / kV;               // lanes per row-direction block: 4 or 8
+  __shared__ __attribute__((aligned(16))) uint8_t tile[kTileCols * kDualPitch];
+  __shared__ __attribute__((aligned(16))) uint32_t ctile[kTileCols];            // [column] -> 4 bytes, one per wave
+  __shared__ __attribute__((aligned(16))) uint8_t rtile[kRowBlocks * kDualRows];  // [block][row]
+  const int tid = threadIdx.x, lane = tid % kWave, w = tid / kWave, h = lane >> 5, c8 = lane & 31;
+
+  // Tile order.  Along the columns first keeps neighbouring workgroups on the same rows of the
+  // input and of the row-wise payload; down the rows first (in runs of 8 tiles per XCD, as in
+  // mx_col_t_kernel) keeps them on the same rows of the transposed payload.  Measured, the first
+  // is faster unless the matrix is wider than tall (16384 x 4096 bf16: 54 vs 63 us; 4096 x
+  // 16384: 59 vs 54 us), so the host picks by shape.
+  const uint32_t row_tiles = (rows + kDualRows - 1) / kDualRows;
+  uint32_t tr, tc;
+  if (cols_first) {
+    const uint32_t col_tiles = (cols + kTileCols - 1) / kTileCols;
+    tr = blockIdx.x / col_tiles;
+    tc = blockIdx.x - tr * col_tiles;
+  } else {
+    uint32_t t = blockIdx.x;
+    if (t < (gridDim.x & ~63u)) {
+      const uint32_t xcd = t & 7u, slot = t >> 3;
+      t = (slot & ~7u) * 8u + xcd * 8u + (slot & 7u);
+    }
+    tc = t / row_tiles;
+    tr = t - tc * row_tiles;
+  }
+  const uint32_t lrow0 = w * 32 + h * 16;                      // first of this lane's 16 rows inside the tile
+  const uint32_t row0 = tr * kDualRows + lrow0, col0 = tc * kTileCols + c8 * kV;
+  const bool active = row0 < rows && col0 < cols;              // rows % 32 == 0 and cols % 32 == 0
+
+  saturate_fp8_conversions();
+  u32x4 v[16];
+  if (active) {
+    const uint8_t* p = static_cast<const uint8_t*>(x) + ((uint64_t)row0 * cols + col0) * kB;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = ld_stream(reinterpret_cast<const u32x4*>(p + (uint64_t)i * cols * kB));
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = u32x4{0u, 0u, 0u, 0u};
+  }
+
+  // ---- blocks down the columns: maxima over this lane's 16 rows, then over both halves
+  u32x4 pm = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    if constexpr (IN == DT_F32) {
+      pm.x = umax(pm.x, absbits_f32(v[i].x)); pm.y = umax(pm.y, absbits_f32(v[i].y));
+      pm.z = umax(pm.z, absbits_f32(v[i].z)); pm.w = umax(pm.w, absbits_f32(v[i].w));
+    } else {
+      pm.x = pk_absmax16(pm.x, v[i].x); pm.y = pk_absmax16(pm.y, v[i].y);
+      pm.z = pk_absmax16(pm.z, v[i].z); pm.w = pk_absmax16(pm.w, v[i].w);
+    }
+  }
+  uint32_t cm[kV];
+  if constexpr (IN == DT_F32) {
+    cm[0] = other_half_max_u32(pm.x); cm[1] = other_half_max_u32(pm.y);
+    cm[2] = other_half_max_u32(pm.z); cm[3] = other_half_max_u32(pm.w);
+  } else {
+    pm.x = other_half_max_pk16(pm.x); pm.y = other_half_max_pk16(pm.y);
+    pm.z = other_half_max_pk16(pm.z); pm.w = other_half_max_pk16(pm.w);
+    if constexpr (IN == DT_BF16) {
+      cm[0] = pm.x << 16; cm[1] = pm.x & 0xFFFF0000u; cm[2] = pm.y << 16; cm[3] = pm.y & 0xFFFF0000u;
+      cm[4] = pm.z << 16; cm[5] = pm.z & 0xFFFF0000u; cm[6] = pm.w << 16; cm[7] = pm.w & 0xFFFF0000u;
+    } else {
+      cm[0] = as_u32(f16_lo(pm.x)); cm[1] = as_u32(f16_hi(pm.x)); cm[2] = as_u32(f16_lo(pm.y)); cm[3] = as_u32(f16_hi(pm.y));
+      cm[4] = as_u32(f16_lo(pm.z)); cm[5] = as_u32(f16_hi(pm.z)); cm[6] = as_u32(f16_lo(pm.w)); cm[7] = as_u32(f16_hi(pm.w));
+    }
+  }
+  // the word that holds column c of row i (fp32: the element itself; 16-bit: it and its neighbour)
+  auto word = [&](int i, int c) -> uint32_t {
+    const int k = IN == DT_F32 ? c : c / 2;
+    return k == 0 ? v[i].x : k == 1 ? v[i].y : k == 2 ? v[i].z : v[i].w;
+  };
+  const uint32_t chunk = (uint32_t)(w * 2 + h);
+#pragma unroll
+  for (int c = 0; c < kV; ++c) {
+    const MxScale<OUT> s = mx_scale_from_absbits<OUT>(cm[c]);
+    uint32_t r[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if constexpr (IN == DT_F32)
+        r[q] = cvt_scaled_4x32<OUT>(word(4 * q, c), word(4 * q + 1, c), word(4 * q + 2, c), word(4 * q + 3, c), s.scale);
+      else
+        r[q] = cvt_scaled_4x16<IN, OUT>(gather_halves(c & 1, word(4 * q, c), word(4 * q + 1, c)),
+                                        gather_halves(c & 1, word(4 * q + 2, c), word(4 * q + 3, c)), s.scale);
+      if (s.nan) r[q] = 0x7F7F7F7Fu;
+    }
+    const uint32_t col = (uint32_t)(c8 * kV + c);
+    *reinterpret_cast<u32x4*>(tile + col * kDualPitch + ((chunk ^ ((col >> 4) & 7u)) << 4)) = u32x4{r[0], r[1], r[2], r[3]};
+    if (h == 0) reinterpret_cast<uint8_t*>(ctile)[col * 4 + w] = (uint8_t)(active ? s.byte : 0u);
+  }
+
+  // ---- blocks along the rows: straight to memory
+  uint32_t rb[4] = {0u, 0u, 0u, 0u};  // this lane's 16 row-scale bytes, rows in byte order
+  uint8_t* drow = data_r + (uint64_t)row0 * cols + col0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    uint32_t m = quad_umax(vec_absmax_bits<IN>(v[i]));
+    if constexpr (LPB == 8) m = umax(m, dpp<kDppRowHalfMirror>(m));
+    const MxScale<OUT> s = mx_scale_from_absbits<OUT>(m);
+    rb[i / 4] |= s.byte << (8 * (i % 4));
+    if (active) {
+      if constexpr (IN == DT_F32) {
+        const uint32_t r = cvt_scaled_4x32<OUT>(v[i].x, v[i].y, v[i].z, v[i].w, s.scale);
+        st_stream(reinterpret_cast<uint32_t*>(drow + (uint64_t)i * cols), s.nan ? 0x7F7F7F7Fu : r);
+      } else {
+        u32x2 r;
+        r.x = cvt_scaled_4x16<IN, OUT>(v[i].x, v[i].y, s.scale);
+        r.y = cvt_scaled_4x16<IN, OUT>(v[i].z, v[i].w, s.scale);
+        if (s.nan) r = u32x2{0x7F7F7F7Fu, 0x7F7F7F7Fu};
+        st_stream(reinterpret_cast<u32x2*>(drow + (uint64_t)i * cols), r);
+      }
+    }
+  }
+  if ((c8 % LPB) == 0)  // inactive lanes hold zero bytes: what the padding of the blocked layout must be
+    *reinterpret_cast<u32x4*>(rtile + (c8 / LPB) * kDualRows + lrow0) = u32x4{rb[0], rb[1], rb[2], rb[3]};
+  __syncthreads();
+
+  // ---- transposed payload: kTileCols output rows (columns of x) x 8 chunks of 16 bytes
+  const uint32_t trow0 = tr * kDualRows, tcol0 = tc * kTileCols;
+#pragma unroll
+  for (int i = 0; i < kTileCols * 8 / kBlock; ++i) {
+    const uint32_t id = tid + i * kBlock, r = id >> 3, q = id & 7;
+    if (tcol0 + r < cols && trow0 + q * 16 < rows) {
+      const u32x4 o = *reinterpret_cast<const u32x4*>(tile + r * kDualPitch + ((q ^ ((r >> 4) & 7u)) << 4));
+      st_stream(reinterpret_cast<u32x4*>(data_c + (uint64_t)(tcol0 + r) * rows + trow0 + q * 16), o);
+    }
+  }
+  // ---- column-block scales [cols, rows/32]: 4 bytes per column of this tile
+  const uint32_t RB = rows / 32, rb0 = tr * 4;
+  if (tid < kTileCols && tcol0 + tid < cols) {
+    const uint32_t sw = ctile[tid];
+    const uint32_t c = tcol0 + tid;
+    if (LAYOUT == DT_SCALE_BLOCKED || (RB % 4 == 0)) {
+      *reinterpret_cast<uint32_t*>(scale_c + scale_offset<LAYOUT>(c, rb0, RB)) = sw;
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (rb0 + k < RB) scale_c[scale_offset<LAYOUT>(c, rb0 + k, RB)] = (uint8_t)(sw >> (8 * k));
+    }
+  }
+  // ---- row-block scales [rows, cols/32]: kRowBlocks bytes per row of this tile
+  const uint32_t KB = cols / 32, kb0 = tc * kRowBlocks;
+  if (tid < kDualRows && trow0 + tid < rows) {
+    const uint32_t r = trow0 + tid;
+#pragma unroll
+    for (int g = 0; g < kRowBlocks / 4; ++g) {
+      uint32_t sw = 0;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) sw |= (uint32_t)rtile[(4 * g + k) * kDualRows + tid] << (8 * k);
+      const uint32_t c = kb0 + 4 * g;
+      if (c >= KB) continue;
+      if (LAYOUT == DT_SCALE_BLOCKED || (KB % 4 == 0)) {
+        *reinterpret_cast<uint32_t*>(scale_r + scale_offset<LAYOUT>(r, c, KB)) = sw;
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (c + k < KB) scale_r[scale_offset<LAYOUT>(r, c + k, KB)] = (uint8_t)(sw >> (8 * k));
+      }
     }
   }
 }

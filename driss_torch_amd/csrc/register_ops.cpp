@@ -232,6 +232,36 @@ std::tuple<Tensor, Tensor> mx_fp8_quantize_ex(const Tensor& input, int64_t block
   return {data, scale};
 }
 
+// Both blockings of one tensor from a single read: (data [M,N], scale [M,N/32]) along the rows and
+// (data [N,M], scale [N,M/32]) down the columns with the payload transposed.  Same checks as
+// mx_fp8_quantize (src/mx_cast.cu:171-219) applied to both dimensions.
+std::tuple<Tensor, Tensor, Tensor, Tensor> mx_fp8_quantize_dual(const Tensor& input, at::ScalarType fp8_type, bool blocked) {
+  TORCH_CHECK(input.is_cuda(), "Input tensor must be a CUDA tensor");
+  TORCH_CHECK(input.is_contiguous(), "Input tensor must be contiguous");
+  TORCH_CHECK(input.scalar_type() == at::kHalf || input.scalar_type() == at::kFloat ||
+                  input.scalar_type() == at::kBFloat16,
+              "Input tensor must be float, half, or bfloat16");
+  TORCH_CHECK(input.dim() == 2, "Only support 2d tensor for now");
+  TORCH_CHECK(fp8_type == at::kFloat8_e4m3fn || fp8_type == at::kFloat8_e5m2,
+              "FP8 type must be Float8_e4m3fn or Float8_e5m2");
+  const int64_t m = input.size(0), n = input.size(1);
+  TORCH_CHECK(m % 32 == 0 && n % 32 == 0, "Need block shape to evenly divide the input tensor for now");
+  Ctx ctx(input);
+  const auto fp8 = input.options().dtype(fp8_type);
+  const auto e8 = input.options().dtype(at::kFloat8_e8m0fnu);
+  Tensor data_r = at::empty({m, n}, fp8), data_c = at::empty({n, m}, fp8);
+  Tensor scale_r = at::empty({blocked ? dt_blocked_scale_bytes(m, n / 32) : m * (n / 32)}, e8);
+  Tensor scale_c = at::empty({blocked ? dt_blocked_scale_bytes(n, m / 32) : n * (m / 32)}, e8);
+  if (input.numel() == 0) return {data_r, scale_r, data_c, scale_c};
+  TORCH_CHECK(reinterpret_cast<std::uintptr_t>(input.data_ptr()) % 16 == 0, "Input tensor must be 16-byte aligned");
+  check_status(dt_mx_fp8_quantize_dual(input.data_ptr(), in_code(input), m, n, out_code(fp8_type),
+                                       blocked ? DT_SCALE_BLOCKED : DT_SCALE_PLAIN, data_r.data_ptr(),
+                                       static_cast<uint8_t*>(scale_r.data_ptr()), data_c.data_ptr(),
+                                       static_cast<uint8_t*>(scale_c.data_ptr()), ctx.stream),
+               "mx_fp8_quantize_dual");
+  return {data_r, scale_r, data_c, scale_c};
+}
+
 std::tuple<Tensor, Tensor> mx_fp8_quantize(Tensor input, int64_t block_size, int64_t axis, bool transpose,
                                            at::ScalarType fp8_type) {
   return mx_fp8_quantize_ex(input, block_size, axis, transpose, fp8_type, false);
@@ -377,6 +407,8 @@ TORCH_LIBRARY(DrissTorch, m) {
       "mx_fp8_quantize_ex(Tensor input, int block_size, int axis, bool transpose, ScalarType fp8_type, bool blocked) -> "
       "(Tensor, Tensor)");
   m.impl("mx_fp8_quantize_ex", c10::DispatchKey::CUDA, TORCH_FN(driss_torch::mx_fp8_quantize_ex));
+  m.def("mx_fp8_quantize_dual(Tensor input, ScalarType fp8_type, bool blocked) -> (Tensor, Tensor, Tensor, Tensor)");
+  m.impl("mx_fp8_quantize_dual", c10::DispatchKey::CUDA, TORCH_FN(driss_torch::mx_fp8_quantize_dual));
   m.def("to_blocked(Tensor scale) -> Tensor");
   m.impl("to_blocked", c10::DispatchKey::CUDA, TORCH_FN(driss_torch::to_blocked));
 }

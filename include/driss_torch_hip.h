@@ -148,6 +148,17 @@ DT_API int dt_mx_fp8_quantize(const void* x, int in_dtype, int64_t rows, int64_t
                               int transpose, int out_dtype, int scale_layout, void* data,
                               uint8_t* scale, dt_stream_t stream);
 
+/* Both blockings of one tensor from a single read: the (axis 1, transpose 0) result in
+ * data_rows [rows, cols] / scale_rows [rows, cols/32] and the (axis 0, transpose 1) result in
+ * data_cols_t [cols, rows] / scale_cols_t [cols, rows/32] -- x for a forward product and x^T
+ * for the weight-gradient product.  Bit-identical to two dt_mx_fp8_quantize calls; rows % 32
+ * == 0 and cols % 32 == 0.  scale_layout applies to both scale matrices.  No counterpart in
+ * the reference, which has the row-wise cast only (src/mx_cast.cu:168-246).               */
+DT_API int dt_mx_fp8_quantize_dual(const void* x, int in_dtype, int64_t rows, int64_t cols,
+                                   int out_dtype, int scale_layout, void* data_rows,
+                                   uint8_t* scale_rows, void* data_cols_t, uint8_t* scale_cols_t,
+                                   dt_stream_t stream);
+
 /* bytes of an [R, C] scale matrix in the blocked layout: 128*ceil(R/128) * 4*ceil(C/4) */
 DT_API int64_t dt_blocked_scale_bytes(int64_t R, int64_t C);
 
