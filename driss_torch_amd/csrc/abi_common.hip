@@ -29,7 +29,9 @@ Knob g_knobs[] = {
     {"mx.row_band4", 1},
     {"gemm.variant", 0},
     {"dynamic.resident", 1},
-    {"dynamic.resident_min_kib", 1024},
+    {"dynamic.resident_min_kib", 0},
+    {"dynamic.resident_gap_lo_kib", 12288},
+    {"dynamic.resident_gap_hi_kib", 40960},
     {"dynamic.resident_spin_limit", 1 << 19},
 };
 constexpr int kNumKnobs = sizeof(g_knobs) / sizeof(g_knobs[0]);

@@ -68,54 +68,6 @@ __device__ __forceinline__ uint32_t pack4_finite(float p0, float p1, float p2, f
   return cvt_pk<OUT, true>(clamp_fp8<OUT>(p2), clamp_fp8<OUT>(p3), w);
 }
 
-// ---- conversions that apply the block scale themselves (v_cvt_scalef32_pk_{fp8,bf8}_{bf16,f16,f32})
-// One instruction turns two inputs into two fp8 bytes of x / 2^(b-127), rounded to nearest even.
-// With MODE.FP16_OVFL set they saturate (infinity included) instead of producing NaN / infinity,
-// which makes them bit-identical to multiply, clamp, convert for every non-NaN input and every
-// scale byte 0..248 (checked exhaustively over all bf16 and f16 patterns and 9 x 65536 fp32
-// patterns per byte on the hardware).  A NaN input gives a NaN code other than 0x7F, so blocks
-// that hold a NaN are still overwritten wholesale by the callers.
-typedef short v2s16 __attribute__((ext_vector_type(2)));
-typedef __bf16 v2bf16 __attribute__((ext_vector_type(2)));
-typedef _Float16 v2f16 __attribute__((ext_vector_type(2)));
-
-// every wave of a kernel that uses them calls this first (the mode register is per wave)
-__device__ __forceinline__ void saturate_fp8_conversions() { __builtin_amdgcn_s_setreg(1 | (23 << 6), 1); }
-
-// two 16-bit inputs packed in one word -> bytes 0-1 (HI false) or 2-3 (HI true) of old
-template <int IN, int OUT, bool HI>
-__device__ __forceinline__ uint32_t cvt_scaled_pair16(uint32_t old, uint32_t pair, float scale) {
-  static_assert(IN == DT_BF16 || IN == DT_F16, "16-bit inputs");
-  const v2s16 o = __builtin_bit_cast(v2s16, old);
-  v2s16 r;
-  if constexpr (IN == DT_BF16) {
-    const v2bf16 x = __builtin_bit_cast(v2bf16, pair);
-    if constexpr (OUT == DT_E5M2) r = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(o, x, scale, HI);
-    else r = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o, x, scale, HI);
-  } else {
-    const v2f16 x = __builtin_bit_cast(v2f16, pair);
-    if constexpr (OUT == DT_E5M2) r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f16(o, x, scale, HI);
-    else r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(o, x, scale, HI);
-  }
-  return __builtin_bit_cast(uint32_t, r);
-}
-template <int OUT, bool HI>
-__device__ __forceinline__ uint32_t cvt_scaled_pair32(uint32_t old, uint32_t a, uint32_t b, float scale) {
-  const v2s16 o = __builtin_bit_cast(v2s16, old);
-  v2s16 r;
-  if constexpr (OUT == DT_E5M2) r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(o, as_f32(a), as_f32(b), scale, HI);
-  else r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(o, as_f32(a), as_f32(b), scale, HI);
-  return __builtin_bit_cast(uint32_t, r);
-}
-// four 16-bit inputs in two words, or four fp32 words -> one word of fp8, all with one scale
-template <int IN, int OUT>
-__device__ __forceinline__ uint32_t cvt_scaled_4x16(uint32_t w0, uint32_t w1, float scale) {
-  return cvt_scaled_pair16<IN, OUT, true>(cvt_scaled_pair16<IN, OUT, false>(w0, w0, scale), w1, scale);
-}
-template <int OUT>
-__device__ __forceinline__ uint32_t cvt_scaled_4x32(uint32_t a, uint32_t b, uint32_t c, uint32_t d, float scale) {
-  return cvt_scaled_pair32<OUT, true>(cvt_scaled_pair32<OUT, false>(a, a, b, scale), c, d, scale);
-}
 // low (half 0) or high (half 1) 16 bits of a and of b as one word {a.half, b.half}
 __device__ __forceinline__ uint32_t gather_halves(int half, uint32_t a, uint32_t b) {
   return __builtin_amdgcn_perm(b, a, half ? 0x07060302u : 0x05040100u);

@@ -163,30 +163,52 @@ inline int launch_amax(const void* x, int64_t numel, void* ws, float* amax_out, 
 // dt_round_mode, bf16 input only); ROUND_SCALE: also round the scale itself (mode 2).
 // CHECK_NAN = false is for callers that know no product can be a NaN (no NaN and no infinity in
 // the tensor, finite scale): the result is the same, without the test.
+//
+// The converts saturate by themselves, so the calling kernel must have executed
+// saturate_fp8_conversions(); bf16-rounded products go to the convert as the packed pairs the
+// rounding instruction leaves.  Per 8 bf16 elements that is 8 unpacks, 8 multiplies, 4 roundings
+// and 4 converts, against 48 instructions with unpacked clamps.
+template <int IN, int OUT, bool ROUND_BF16>
+__device__ __forceinline__ void products_to_fp8(const float (&p)[InTraits<IN>::kVec], uint32_t (&r)[InTraits<IN>::kVec / 4],
+                                                float cvt_scale) {
+  if constexpr (IN == DT_F32 || !ROUND_BF16) {
+#pragma unroll
+    for (int q = 0; q < InTraits<IN>::kVec / 4; ++q)
+      r[q] = cvt_scaled_4x32<OUT>(as_u32(p[4 * q]), as_u32(p[4 * q + 1]), as_u32(p[4 * q + 2]), as_u32(p[4 * q + 3]), cvt_scale);
+  } else {
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+      r[q] = cvt_scaled_4x16<DT_BF16, OUT>(pack_bf16x2(p[4 * q], p[4 * q + 1]), pack_bf16x2(p[4 * q + 2], p[4 * q + 3]), cvt_scale);
+  }
+}
+template <int IN>
+__device__ __forceinline__ void products_of(u32x4 w, float s, float (&p)[InTraits<IN>::kVec]) {
+  if constexpr (IN == DT_F32) {
+    p[0] = as_f32(w.x) * s; p[1] = as_f32(w.y) * s; p[2] = as_f32(w.z) * s; p[3] = as_f32(w.w) * s;
+  } else {
+    p[0] = bf16_lo(w.x) * s; p[1] = bf16_hi(w.x) * s; p[2] = bf16_lo(w.y) * s; p[3] = bf16_hi(w.y) * s;
+    p[4] = bf16_lo(w.z) * s; p[5] = bf16_hi(w.z) * s; p[6] = bf16_lo(w.w) * s; p[7] = bf16_hi(w.w) * s;
+  }
+}
+
 template <int IN, int OUT, bool ROUND_BF16, bool CHECK_NAN = true>
 __device__ __forceinline__ void cast_vec(u32x4 w, float s, uint8_t* __restrict__ out, int64_t vec_index) {
-  if constexpr (IN == DT_F32) {
-    const float p0 = as_f32(w.x) * s, p1 = as_f32(w.y) * s, p2 = as_f32(w.z) * s, p3 = as_f32(w.w) * s;
-    st_stream(reinterpret_cast<uint32_t*>(out) + vec_index,
-              CHECK_NAN ? pack4<OUT>(p0, p1, p2, p3) : pack4_clamped<OUT>(p0, p1, p2, p3));
-  } else {
-    float p[8] = {bf16_lo(w.x) * s, bf16_hi(w.x) * s, bf16_lo(w.y) * s, bf16_hi(w.y) * s,
-                  bf16_lo(w.z) * s, bf16_hi(w.z) * s, bf16_lo(w.w) * s, bf16_hi(w.w) * s};
-    if constexpr (ROUND_BF16) {
-      round2_to_bf16(p[0], p[1]); round2_to_bf16(p[2], p[3]);
-      round2_to_bf16(p[4], p[5]); round2_to_bf16(p[6], p[7]);
+  constexpr int kV = InTraits<IN>::kVec;
+  float p[kV];
+  products_of<IN>(w, s, p);
+  uint32_t r[kV / 4];
+  products_to_fp8<IN, OUT, ROUND_BF16>(p, r, 1.0f);
+  if constexpr (CHECK_NAN) {  // rounding to bf16 keeps a NaN a NaN and its sign
+    bool any_nan = false;
+#pragma unroll
+    for (int k = 0; k < kV; k += 2) any_nan |= __builtin_isunordered(p[k], p[k + 1]);
+    if (__builtin_expect(any_nan, 0)) {
+#pragma unroll
+      for (int q = 0; q < kV / 4; ++q) r[q] = nan_patch4(r[q], p[4 * q], p[4 * q + 1], p[4 * q + 2], p[4 * q + 3]);
     }
-    u32x2 r;
-    r.x = pack4_clamped<OUT>(p[0], p[1], p[2], p[3]);
-    r.y = pack4_clamped<OUT>(p[4], p[5], p[6], p[7]);
-    const bool any_nan = (p[0] != p[0]) | (p[1] != p[1]) | (p[2] != p[2]) | (p[3] != p[3]) | (p[4] != p[4]) |
-                         (p[5] != p[5]) | (p[6] != p[6]) | (p[7] != p[7]);
-    if (CHECK_NAN && __builtin_expect(any_nan, 0)) {
-      r.x = nan_patch4(r.x, p[0], p[1], p[2], p[3]);
-      r.y = nan_patch4(r.y, p[4], p[5], p[6], p[7]);
-    }
-    st_stream(reinterpret_cast<u32x2*>(out) + vec_index, r);
   }
+  if constexpr (IN == DT_F32) st_stream(reinterpret_cast<uint32_t*>(out) + vec_index, r[0]);
+  else st_stream(reinterpret_cast<u32x2*>(out) + vec_index, u32x2{r[0], r[1]});
 }
 
 template <int IN, int OUT, bool ROUND_BF16>
@@ -208,6 +230,7 @@ __global__ __launch_bounds__(kBlock) void cast_kernel(const void* __restrict__ x
                                                       uint8_t* __restrict__ out2) {
   constexpr int kV = InTraits<IN>::kVec;
   constexpr int OUT2 = OUT == DT_E4M3FN ? DT_E5M2 : DT_E4M3FN;
+  saturate_fp8_conversions();
   float s = scale[0], s2 = PAIR ? scale[1] : 0.f;
   if constexpr (ROUND_SCALE) { s = round_to_bf16(s); s2 = round_to_bf16(s2); }
   const u32x4* v = static_cast<const u32x4*>(x);

@@ -36,30 +36,16 @@ constexpr size_t kWsTimeout = 196; // u32, set (and left set) if a barrier wait 
 // One vector to e4m3fn and e5m2 at once, for products that cannot be NaN.  The two scales are
 // fmax / amax with fmax = 448 and 57344 = 128 * 448, so scale_e5m2 == 128 * scale_e4m3 exactly
 // (a power of two commutes with every rounding on the way, also with the bf16 roundings of
-// modes 1 and 2, and with the clamp): the e5m2 operand is the clamped e4m3 operand times 128.
+// modes 1 and 2): the e5m2 bytes come from the same products, converted with a scale of 2^-7.
 template <int IN, bool ROUND_BF16>
 __device__ __forceinline__ void cast_vec_pair_finite(u32x4 w, float s4, uint8_t* __restrict__ out4,
                                                      uint8_t* __restrict__ out5, uint32_t vec_index) {
   constexpr int kV = InTraits<IN>::kVec;
   float p[kV];
-  if constexpr (IN == DT_F32) {
-    p[0] = as_f32(w.x) * s4; p[1] = as_f32(w.y) * s4; p[2] = as_f32(w.z) * s4; p[3] = as_f32(w.w) * s4;
-  } else {
-    p[0] = bf16_lo(w.x) * s4; p[1] = bf16_hi(w.x) * s4; p[2] = bf16_lo(w.y) * s4; p[3] = bf16_hi(w.y) * s4;
-    p[4] = bf16_lo(w.z) * s4; p[5] = bf16_hi(w.z) * s4; p[6] = bf16_lo(w.w) * s4; p[7] = bf16_hi(w.w) * s4;
-    if constexpr (ROUND_BF16) {
-      round2_to_bf16(p[0], p[1]); round2_to_bf16(p[2], p[3]);
-      round2_to_bf16(p[4], p[5]); round2_to_bf16(p[6], p[7]);
-    }
-  }
+  products_of<IN>(w, s4, p);
   uint32_t r4[kV / 4], r5[kV / 4];
-#pragma unroll
-  for (int q = 0; q < kV / 4; ++q) {
-    const float c0 = clamp_fp8<DT_E4M3FN>(p[4 * q]), c1 = clamp_fp8<DT_E4M3FN>(p[4 * q + 1]);
-    const float c2 = clamp_fp8<DT_E4M3FN>(p[4 * q + 2]), c3 = clamp_fp8<DT_E4M3FN>(p[4 * q + 3]);
-    r4[q] = cvt_pk<DT_E4M3FN, true>(c2, c3, cvt_pk<DT_E4M3FN, false>(c0, c1, 0u));
-    r5[q] = cvt_pk<DT_E5M2, true>(c2 * 128.0f, c3 * 128.0f, cvt_pk<DT_E5M2, false>(c0 * 128.0f, c1 * 128.0f, 0u));
-  }
+  products_to_fp8<IN, DT_E4M3FN, ROUND_BF16>(p, r4, 1.0f);
+  products_to_fp8<IN, DT_E5M2, ROUND_BF16>(p, r5, 0x1p-7f);  // the convert divides by its scale: x 128
   if constexpr (IN == DT_F32) {
     st_stream(reinterpret_cast<uint32_t*>(out4) + vec_index, r4[0]);
     st_stream(reinterpret_cast<uint32_t*>(out5) + vec_index, r5[0]);
@@ -79,6 +65,7 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
   constexpr int OUT2 = OUT == DT_E4M3FN ? DT_E5M2 : DT_E4M3FN;
   extern __shared__ __attribute__((aligned(16))) u32x4 keep[];  // [kResLdsVecs][kBlock]
   __shared__ uint32_t red[kBlock / kWave];
+  saturate_fp8_conversions();
   __shared__ uint32_t bcast;
   const int tid = threadIdx.x;
   const u32x4* v = static_cast<const u32x4*>(x);
@@ -108,9 +95,14 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
   };
   constexpr int kResBatch = 16;
   static_assert(kResRegVecs % 4 == 0 && kResLdsVecs % 4 == 0, "batches");
+  // Vector slots k >= nk lie past the end for every lane of this workgroup: a tensor smaller than
+  // the chip's capacity skips whole batches (a branch the workgroup takes as one), in both passes.
+  const uint32_t block_first = blockIdx.x * kBlock;
+  const uint32_t nk = block_first < (uint32_t)nvec ? ((uint32_t)nvec - block_first + (uint32_t)stride - 1u) / (uint32_t)stride : 0u;
   // the LDS part first (through a batch of registers), then the register part in place
 #pragma unroll
   for (int b = 0; b < kResLdsVecs; b += kResBatch) {
+    if ((uint32_t)(kResRegVecs + b) >= nk) break;
     u32x4 t[kResBatch];
 #pragma unroll
     for (int j = 0; j < kResBatch; ++j)
@@ -126,6 +118,7 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
   }
 #pragma unroll
   for (int b = 0; b < kResRegVecs; b += kResBatch) {
+    if ((uint32_t)b >= nk) break;
 #pragma unroll
     for (int j = 0; j < kResBatch; ++j)
       if (b + j < kResRegVecs) r[b + j] = fetch(b + j);
@@ -233,9 +226,19 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
       }
     };
 #pragma unroll
-    for (int k = 0; k < kResRegVecs; ++k) emit(k, r[k]);
+    for (int b = 0; b < kResRegVecs; b += kResBatch) {
+      if ((uint32_t)b >= nk) break;
 #pragma unroll
-    for (int k = 0; k < kResLdsVecs; ++k) emit(kResRegVecs + k, keep[k * kBlock + tid]);
+      for (int j = 0; j < kResBatch; ++j)
+        if (b + j < kResRegVecs) emit(b + j, r[b + j]);
+    }
+#pragma unroll
+    for (int b = 0; b < kResLdsVecs; b += kResBatch) {
+      if ((uint32_t)(kResRegVecs + b) >= nk) break;
+#pragma unroll
+      for (int j = 0; j < kResBatch; ++j)
+        if (b + j < kResLdsVecs) emit(kResRegVecs + b + j, keep[(b + j) * kBlock + tid]);
+    }
   }
   if (blockIdx.x == 0 && tid < tail) {
     const int64_t e = nvec * kV + tid;
@@ -331,7 +334,12 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
 template <bool PAIR>
 inline int launch_resident(const void* x, int in_dtype, int64_t numel, int out_dtype, int round_mode, void* ws, void* out,
                            void* out2, float* amax_out, float* scale_out, float fmax0, float fmax1, hipStream_t stream) {
-  if (!tuning("dynamic.resident") || numel * (in_dtype == DT_F32 ? 4 : 2) < (int64_t)tuning("dynamic.resident_min_kib") * 1024)
+  // Where the two kernels win: between about 12 and 40 MiB the cast's second read of x comes out
+  // of the 256 MiB last-level cache faster than this kernel's barrier costs (32 MiB bf16: 17.0 vs
+  // 18.4 us).  Below, one launch beats two; above, the second read goes to HBM (128 MiB: 50 vs 61 us).
+  const int64_t bytes = numel * (in_dtype == DT_F32 ? 4 : 2);
+  if (!tuning("dynamic.resident") || bytes < (int64_t)tuning("dynamic.resident_min_kib") * 1024) return kResidentNotTaken;
+  if (bytes >= (int64_t)tuning("dynamic.resident_gap_lo_kib") * 1024 && bytes < (int64_t)tuning("dynamic.resident_gap_hi_kib") * 1024)
     return kResidentNotTaken;
 #define DT_RES(IN, OUT, RB, RS) \
   return launch_resident_impl<IN, OUT, RB, RS, PAIR>(x, numel, ws, out, out2, amax_out, scale_out, fmax0, fmax1, stream)

@@ -18,6 +18,7 @@ __global__ __launch_bounds__(kBlock) void rowwise_wave_kernel(const void* __rest
                                                               float* __restrict__ amax_out,
                                                               float* __restrict__ scale_out) {
   constexpr int kV = InTraits<IN>::kVec;
+  saturate_fp8_conversions();
   const int lane = threadIdx.x % kWave;
   const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
   if (row >= rows) return;  // whole wave leaves together; the kernel has no barrier
@@ -61,6 +62,7 @@ __global__ __launch_bounds__(kBlock) void rowwise_block_kernel(const void* __res
                                                                float* __restrict__ amax_out,
                                                                float* __restrict__ scale_out) {
   constexpr int kB = InTraits<IN>::kBytes, kV = InTraits<IN>::kVec;
+  saturate_fp8_conversions();
   __shared__ uint32_t lds[kBlock / kWave];
   const int64_t row = blockIdx.x;
   const uint8_t* xrow = static_cast<const uint8_t*>(x) + row * cols * kB;

@@ -18,8 +18,10 @@ MODE = {1: "ROUND_V1", 2: "ROUND_V2", 3: "ROUND_V3"}
 def cabi(gpu_device):
     from driss_torch_amd import cabi as c
 
-    keep = {k: c.get_tuning(k) for k in ("dynamic.resident", "dynamic.resident_min_kib", "dynamic.resident_spin_limit")}
+    keep = {k: c.get_tuning(k) for k in ("dynamic.resident", "dynamic.resident_min_kib", "dynamic.resident_gap_lo_kib",
+                                         "dynamic.resident_gap_hi_kib", "dynamic.resident_spin_limit")}
     c.set_tuning("dynamic.resident_min_kib", 0)  # every size takes the resident kernel
+    c.set_tuning("dynamic.resident_gap_hi_kib", 0)
     yield c
     for k, v in keep.items():
         c.set_tuning(k, v)
