@@ -256,6 +256,17 @@ def extra_kernels(torch, cabi, util, dev, K, W, gemm_only=False):
                 lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
                            torch.empty((8192, 256), dtype=torch.uint8, device=dev)),
                 lambda x, dd, s: cabi.mx_fp8_quantize(x, 1, False, e4, cabi.SCALE_PLAIN, dd, s))
+        nblk = cabi.lib().dt_blocked_scale_bytes(8192, 256)
+        hbm_row("mx_fp8_quantize rows, blocked scales", "config 4: bf16 [8192,8192], scales in the GEMM's layout", mxb,
+                lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
+                           torch.empty((nblk,), dtype=torch.uint8, device=dev)),
+                lambda x, dd, s: cabi.mx_fp8_quantize(x, 1, False, e4, cabi.SCALE_BLOCKED, dd, s))
+        hbm_row("mx_fp8_quantize_dual (rows + transposed columns from one read)",
+                "config 4: bf16 [8192,8192], blocked scales", n * 2 + 2 * (n + n // 32),
+                lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
+                           torch.empty((nblk,), dtype=torch.uint8, device=dev), torch.empty((8192, 8192), dtype=e4, device=dev),
+                           torch.empty((nblk,), dtype=torch.uint8, device=dev)),
+                lambda x, dr, sr, dc, sc: cabi.mx_fp8_quantize_dual(x, e4, cabi.SCALE_BLOCKED, (dr, sr, dc, sc)))
         hbm_row("mx_fp8_quantize cols (transposed out)", "config 4: bf16 [8192,8192], blocks down columns", mxb,
                 lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
                            torch.empty((8192, 256), dtype=torch.uint8, device=dev)),

@@ -200,16 +200,16 @@ def mx_fp8_quantize(x: torch.Tensor, axis: int = 1, transpose: bool = False, out
     return data, scale
 
 
-def mx_fp8_quantize_dual(x: torch.Tensor, out_dtype: torch.dtype = torch.float8_e4m3fn, layout: int = SCALE_PLAIN):
+def mx_fp8_quantize_dual(x: torch.Tensor, out_dtype: torch.dtype = torch.float8_e4m3fn, layout: int = SCALE_PLAIN, outs=None):
     """(data_rows, scale_rows, data_cols_t, scale_cols_t): the (axis 1) cast of x and the (axis 1) cast of x^T
-    from one read of x."""
+    from one read of x.  `outs`: the four output tensors, to reuse them."""
     R, Cc = x.shape
-    dr_shape, sr_shape = mx_shapes(R, Cc, 1, False, layout)
-    dc_shape, sc_shape = mx_shapes(R, Cc, 0, True, layout)
-    dr = torch.empty(dr_shape, dtype=out_dtype, device=x.device)
-    sr = torch.empty(sr_shape, dtype=torch.uint8, device=x.device)
-    dc = torch.empty(dc_shape, dtype=out_dtype, device=x.device)
-    sc = torch.empty(sc_shape, dtype=torch.uint8, device=x.device)
+    if outs is None:
+        dr_shape, sr_shape = mx_shapes(R, Cc, 1, False, layout)
+        dc_shape, sc_shape = mx_shapes(R, Cc, 0, True, layout)
+        outs = (torch.empty(dr_shape, dtype=out_dtype, device=x.device), torch.empty(sr_shape, dtype=torch.uint8, device=x.device),
+                torch.empty(dc_shape, dtype=out_dtype, device=x.device), torch.empty(sc_shape, dtype=torch.uint8, device=x.device))
+    dr, sr, dc, sc = outs
     _check(lib().dt_mx_fp8_quantize_dual(x.data_ptr(), IN_DTYPE[x.dtype], R, Cc, OUT_DTYPE[out_dtype], layout, dr.data_ptr(),
                                          sr.data_ptr(), dc.data_ptr(), sc.data_ptr(), _stream()), "dt_mx_fp8_quantize_dual")
     return dr, sr, dc, sc

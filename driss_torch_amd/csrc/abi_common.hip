@@ -15,9 +15,12 @@ struct Knob {
 };
 // Launch-shape knobs.  Workgroups per CU for the persistent grids, chosen on MI355X.
 //   dynamic.resident: 1 = per-tensor dynamic quantization of a tensor that fits the chip runs as one
-//                 kernel that keeps it in registers and LDS; dynamic.resident_min_kib = smallest such tensor
+//                 kernel that keeps it in registers and LDS; dynamic.resident_min_kib = smallest such
+//                 tensor; sizes in [resident_gap_lo_kib, resident_gap_hi_kib) take the two kernels
+//   mx.dual:      1 = dt_mx_fp8_quantize_dual reads x once (0: two single casts)
+//   mx.row_band4: 1 = row-wise MX cast with blocked scales walks 4 rows x 512 elements per wave pass
 //   gemm.variant: 0 = pick the tile by problem size, 1 = 128x128 tiles, 2 = 256x256 tiles,
-//                 7 = 256x256 tiles without the L2 prefetch loads
+//                 7 = 256x256 tiles without the L2 prefetch loads, 8 = 256x256 tiles on 8 waves (e4m3 only)
 Knob g_knobs[] = {
     {"amax.blocks_per_cu", 1},
     {"amax.stream_before_cast", 0},

@@ -164,7 +164,7 @@ def test_mx_gemm_reference_sizes(d, size, dist):
     _check_gemm(d, M, K, N, 600 + M + N, dist)
 
 
-@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("variant", [1, 2, 8])
 @pytest.mark.parametrize("size", [(128, 128, 128), (512, 256, 640), (133, 512, 528), (300, 1024, 264)])
 def test_mx_gemm_both_tile_shapes(d, cabi, variant, size):
     cabi.set_tuning("gemm.variant", variant)
