@@ -118,6 +118,38 @@ def test_saturated_cast_modes_signed_and_special(d, in_dtype, fp8_dtype, mode):
     assert torch.equal(util.codes(got), co.saturated_cast(a, (scale * 8).item(), fp8_dtype, mode))
 
 
+@pytest.mark.parametrize("fp8_dtype", FP8)
+def test_saturated_cast_every_bf16_pattern(d, fp8_dtype):
+    """all 65536 bf16 bit patterns (NaNs of both signs, infinities, subnormals) under every rounding
+    mode and scales that put the products below, inside and beyond the fp8 range"""
+    a = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).reshape(256, 256)
+    ag = a.cuda()
+    for scale in (1.0, 0.37, 448.0 / 3.0, 57344.0, 1e-3, 2.0**-20, 3.0e38):
+        sg = torch.tensor([scale], device="cuda")
+        for mode in (1, 2, 3):
+            got = d.saturated_cast_mode(ag, sg, fp8_dtype, mode)
+            assert torch.equal(util.codes(got), co.saturated_cast(a, scale, fp8_dtype, mode)), (scale, mode)
+
+
+@pytest.mark.parametrize("fp8_dtype", FP8)
+def test_saturated_cast_fp32_bit_pattern_sweep(d, fp8_dtype):
+    """2^20 fp32 patterns: every exponent with random mantissas, plus the neighbourhood of every fp8
+    rounding boundary (midpoints between representable values, +- 1 ulp)"""
+    g = util.gen(9)
+    bits = torch.randint(0, 2**31 - 1, (1 << 20,), generator=g, dtype=torch.int64)
+    bits = bits | (torch.randint(0, 2, (1 << 20,), generator=g, dtype=torch.int64) << 31)
+    x = bits.to(torch.uint32).view(torch.float32)
+    codes = torch.arange(256, dtype=torch.uint8).view(fp8_dtype).float()
+    vals = codes[torch.isfinite(codes)].unique()
+    mids = ((vals[:-1].double() + vals[1:].double()) / 2).float()
+    near = torch.cat([mids, torch.nextafter(mids, torch.tensor(float("inf"))), torch.nextafter(mids, torch.tensor(-float("inf"))), vals])
+    x = torch.cat([x, near, near * 0.5, near * 3.0])
+    x = x[: x.numel() // 4 * 4].reshape(-1, 4).contiguous()
+    for scale in (1.0, 2.0, 1.0 / 3.0):
+        got = d.saturated_cast_mode(x.cuda(), torch.tensor([scale], device="cuda"), fp8_dtype, 3)
+        assert torch.equal(util.codes(got), co.saturated_cast(x, scale, fp8_dtype, co.ROUND_V3)), scale
+
+
 def test_saturated_cast_reference_edge_vector(d):
     """test/test_sat_cast.py:66-83: 0.3223 * 57344 -> e5m2 is 20480 with single rounding; the
     rank-1 scale of that test selects it, a 0-dim scale reproduces eager's 16384."""
