@@ -140,3 +140,26 @@ def test_row_cast_blocked_scales_four_row_pass(d, cabi, shape, in_dtype):
             cabi.set_tuning("mx.row_band4", band4)
             data, scale = d.mx_fp8_quantize_blocked(g, 1, out_dtype)
             assert torch.equal(util.codes(data), rd) and torch.equal(util.codes(scale), co.to_blocked(rs))
+
+
+@pytest.mark.parametrize("out_dtype", [E4, E5])
+def test_mx_casts_every_bf16_pattern(d, out_dtype):
+    """all 65536 bf16 bit patterns, once with 32 neighbouring patterns per block (every block
+    magnitude from subnormal to infinity, NaN blocks) and once shuffled, through the row, column,
+    transposed-column and one-read kernels"""
+    pats = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    perm = torch.randperm(65536, generator=util.gen(4))
+    for x in (pats.reshape(2048, 32), pats.reshape(32, 2048).t().contiguous(), pats[perm].reshape(256, 256)):
+        g = x.cuda()
+        rd, rs = co.mx_quantize(x, axis=1, transpose=False, out_dtype=out_dtype)
+        data, scale = d.mx_fp8_quantize(g, 32, 1, False, out_dtype)
+        assert torch.equal(util.codes(data), rd) and torch.equal(util.codes(scale), rs.flatten())
+        if x.shape[0] % 32 == 0:
+            cd, cs = co.mx_quantize(x, axis=0, transpose=True, out_dtype=out_dtype)
+            data, scale = d.mx_fp8_quantize(g, 32, 0, True, out_dtype)
+            assert torch.equal(util.codes(data), cd) and torch.equal(util.codes(scale), cs.flatten())
+            data, scale = d.mx_fp8_quantize(g, 32, 0, False, out_dtype)
+            assert torch.equal(util.codes(data), cd.t()) and torch.equal(util.codes(scale).view(cs.shape[1], cs.shape[0]), cs.t())
+            dr, sr, dc, sc = d.mx_fp8_quantize_dual(g, out_dtype)
+            assert torch.equal(util.codes(dr), rd) and torch.equal(util.codes(sr), rs.flatten())
+            assert torch.equal(util.codes(dc), cd) and torch.equal(util.codes(sc), cs.flatten())
