@@ -83,3 +83,39 @@ def test_mx_quantize_blocked_and_gemm_compile(d):
 def test_to_blocked_compile(d):
     s = torch.randint(0, 255, (256, 12), dtype=torch.uint8, device="cuda")
     _same(_compiled(d.to_blocked)(s), d.to_blocked(s))
+
+
+def test_ops_replay_from_a_captured_graph(d):
+    """every op recorded once into a HIP graph and replayed with new input contents, with eager
+    calls and synchronisations between the replays; each replay equals the eager results bit for bit
+    (per-tensor dynamic quantization takes its two-kernel path under capture)"""
+    M, K, N = 512, 1024, 256
+    sx = util.normal_with_outliers((M, K), 100).cuda()
+    sw = util.normal((N, K), 101).cuda()
+    scale = torch.tensor([3.7], device="cuda")
+
+    def run(x, w):
+        a, sa = d.mx_fp8_quantize_blocked(x)
+        b, sb = d.mx_fp8_quantize_blocked(w)
+        return (d.amax(x), d.saturated_cast(x, scale, E4), d.dynamic_scaled_quant(x, E5),
+                d.dynamic_scaled_quant_pair(x), d.dynamic_scaled_quant_rowwise(x, E4), d.mx_fp8_quantize(x),
+                d.mx_fp8_quantize(x, 32, 0, True), d.mx_fp8_quantize_dual(x, E4, True), d.mx_fp8_bf16(a, b.t(), sa, sb))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(sx, sw)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = run(sx, sw)
+    for seed in (102, 103, 104):
+        x = util.normal_with_outliers((M, K), seed).cuda()
+        w = util.normal((N, K), seed + 10).cuda()
+        sx.copy_(x)
+        sw.copy_(w)
+        graph.replay()
+        torch.cuda.synchronize()
+        _same(captured, run(x, w))
+        torch.cuda.synchronize()
