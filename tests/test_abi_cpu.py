@@ -56,6 +56,14 @@ def test_host_validation_without_gpu():
     assert L.dt_mx_fp8_quantize(fake, cabi.BF16, 32, 128, 2, 0, cabi.E4M3FN, 0, fake, fake, None) == 6
     assert L.dt_mx_fp8_quantize(fake, cabi.BF16, 32, 128, 0, 0, cabi.E4M3FN, 1, fake, fake, None) == 6  # blocked needs [outer, inner/32]
     assert L.dt_mx_fp8_quantize(fake, cabi.BF16, 0, 128, 1, 0, cabi.E4M3FN, 0, None, None, None) == 0
+    # both blockings at once: both dimensions are blocked
+    assert L.dt_mx_fp8_quantize_dual(fake, cabi.BF16, 128, 48, cabi.E4M3FN, 0, fake, fake, fake, fake, None) == 2
+    assert L.dt_mx_fp8_quantize_dual(fake, cabi.BF16, 48, 128, cabi.E4M3FN, 0, fake, fake, fake, fake, None) == 2
+    assert L.dt_mx_fp8_quantize_dual(fake, cabi.BF16, 128, 128, cabi.E4M3FN, 2, fake, fake, fake, fake, None) == 6
+    assert L.dt_mx_fp8_quantize_dual(fake, 9, 128, 128, cabi.E4M3FN, 0, fake, fake, fake, fake, None) == 1
+    assert L.dt_mx_fp8_quantize_dual(fake, cabi.BF16, 128, 128, cabi.E4M3FN, 0, fake, fake, None, fake, None) == 3
+    assert L.dt_mx_fp8_quantize_dual(fake + 1, cabi.BF16, 128, 128, cabi.E4M3FN, 0, fake, fake, fake, fake, None) == 4
+    assert L.dt_mx_fp8_quantize_dual(None, cabi.BF16, 0, 128, cabi.E4M3FN, 0, None, None, None, None, None) == 0
     assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 128, 128, 96, 96, 96, fake, 128, None) == 2  # K % 128
     assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 128, 126, 128, 128, 128, fake, 126, None) == 2  # N % 4
     assert L.dt_mx_fp8_bf16(fake + 8, fake, fake, fake, 128, 128, 128, 128, 128, fake, 128, None) == 4
@@ -128,6 +136,9 @@ def test_fake_impls_cover_every_op():
         assert data.shape == (384, 256) and scale.shape == (384 * 8,)
         data, scale = d.mx_fp8_quantize_blocked(x)
         assert scale.shape == (256 * 12,)
+        dr, sr, dc, sc = d.mx_fp8_quantize_dual(x, torch.float8_e5m2, True)
+        assert dr.shape == (256, 384) and dc.shape == (384, 256) and dr.dtype == dc.dtype == torch.float8_e5m2
+        assert sr.shape == (256 * 12,) and sc.shape == (384 * 8,) and sc.dtype == torch.float8_e8m0fnu
         a8 = torch.empty(256, 384, dtype=torch.float8_e4m3fn, device="cuda")
         b8 = torch.empty(128, 384, dtype=torch.float8_e4m3fn, device="cuda").t()
         out = d.mx_fp8_bf16(a8, b8, scale, scale)
