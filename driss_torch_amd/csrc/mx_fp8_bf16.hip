@@ -48,7 +48,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const uint8_t* __restrict__ sfa,
     const uint8_t* __restrict__ sfb, int M, int N, int K, int64_t lda, int64_t ldb, uint16_t* __restrict__ out,
     int64_t ldo, int tiles_m, int tiles_n, int wide_stores) {
-  constexpr int kThreads = WAVES_M * WAVES_N * kWave;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
   constexpr int TM = WM / 16, TN = WN / 16;            // MFMA tiles per wave
   constexpr int KC = FP4 ? 2 : 1;                      // 128-element MFMAs (and blocked scale chunks) per K-step

@@ -480,7 +480,6 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
                                                          uint8_t* __restrict__ data_r, uint8_t* __restrict__ scale_r,
                                                          uint8_t* __restrict__ data_c, uint8_t* __restrict__ scale_c, int cols_first) {
   constexpr int kV = InTraits<IN>::kVec;     // columns per lane: 8 or 4
-  constexpr int kW = kV / 4;                 // fp8 words per lane and row
   constexpr int kB = InTraits<IN>::kBytes;
   constexpr int kTileCols = 32 * kV;         // 256 or 128
   constexpr int kRowBlocks = kTileCols / 32; // row-direction blocks per tile row: 8 or 4
