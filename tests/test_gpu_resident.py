@@ -161,3 +161,21 @@ def test_resident_wait_gives_up_loudly(cabi):
     ref, ramax, _ = co.dynamic_scaled_quant(x.cpu(), E4, co.ROUND_V2)
     assert torch.equal(util.codes(out), ref) and amax.item() == ramax.item()
     assert _timeout_flag(cabi) == 0
+
+
+@pytest.mark.parametrize("slots,delta", [(1, 3), (15, -8), (16, 0), (16, 13), (17, -3), (33, 5), (92, 0), (92, 8), (93, -1), (108, 7), (109, 1)],
+                         ids=lambda v: str(v))
+def test_resident_batch_boundaries(cabi, slots, delta):
+    """sizes around the 16-vector batches a workgroup may skip, around the register / LDS split (92
+    vectors per lane) and with a ragged tail: a lane holds `slots` vectors, give or take a few elements"""
+    cabi.set_tuning("dynamic.resident", 1)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    numel = slots * cus * 256 * 8 + delta
+    x = util.normal_with_outliers((1, numel), 40 + slots, torch.bfloat16)
+    x[0, -1] = 4096.0  # the maximum sits in the last (possibly partial) vector
+    o4, o5, amax, scales = cabi.dynamic_scaled_quant_pair(x.cuda(), 2)
+    r4, ramax, rs4 = co.dynamic_scaled_quant(x, E4, co.ROUND_V2)
+    r5, _, rs5 = co.dynamic_scaled_quant(x, E5, co.ROUND_V2)
+    assert amax.item() == ramax.item() == 4096.0 and scales.tolist() == [rs4.item(), rs5.item()]
+    assert torch.equal(util.codes(o4), r4) and torch.equal(util.codes(o5), r5)
+    assert _timeout_flag(cabi) == 0
