@@ -26,6 +26,7 @@ Knob g_knobs[] = {
     {"amax.stream_before_cast", 0},
     {"cast.blocks_per_cu", 2},
     {"cast.pair_blocks_per_cu", 3},
+    {"cast.pair_alone_blocks_per_cu", 1},
     {"mx.blocks_per_cu", 16},
     {"mx.col_blocks_per_cu", 16},
     {"mx.dual", 1},
