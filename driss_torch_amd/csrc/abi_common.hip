@@ -27,7 +27,7 @@ Knob g_knobs[] = {
     {"cast.blocks_per_cu", 2},
     {"cast.pair_blocks_per_cu", 3},
     {"cast.pair_alone_blocks_per_cu", 1},
-    {"mx.blocks_per_cu", 16},
+    {"mx.blocks_per_cu", 32},
     {"mx.col_blocks_per_cu", 16},
     {"mx.dual", 1},
     {"mx.row_band4", 1},
