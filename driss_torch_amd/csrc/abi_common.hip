@@ -25,8 +25,7 @@ Knob g_knobs[] = {
     {"amax.blocks_per_cu", 1},
     {"amax.stream_before_cast", 0},
     {"cast.blocks_per_cu", 2},
-    {"cast.pair_blocks_per_cu", 3},
-    {"cast.pair_alone_blocks_per_cu", 1},
+    {"cast.pair_blocks_per_cu", 2},
     {"mx.blocks_per_cu", 32},
     {"mx.col_blocks_per_cu", 16},
     {"mx.dual", 1},

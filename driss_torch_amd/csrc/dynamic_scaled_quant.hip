@@ -65,7 +65,7 @@ extern "C" int dt_dynamic_scaled_quant_pair(const void* x, int in_dtype, int64_t
     return DT_OK;
   if (int st = dt_amax_scales(x, in_dtype, numel, amax_out, scale_out, workspace, workspace_bytes, stream)) return st;
   const float* scale = reinterpret_cast<const float*>(static_cast<const uint8_t*>(workspace) + dt::kWsScale);
-  return dt::launch_cast<true>(x, in_dtype, numel, scale, DT_E4M3FN, round_mode, out_e4m3fn, out_e5m2, dt::as_hip(stream), true);
+  return dt::launch_cast<true>(x, in_dtype, numel, scale, DT_E4M3FN, round_mode, out_e4m3fn, out_e5m2, dt::as_hip(stream));
 }
 
 extern "C" int dt_dynamic_scaled_quant_rowwise(const void* x, int in_dtype, int64_t rows, int64_t cols, int out_dtype,

@@ -275,17 +275,18 @@ __global__ __launch_bounds__(kBlock) void cast_kernel_unaligned(const void* __re
 
 template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR>
 inline int launch_cast_impl(const void* x, int64_t numel, const float* scale, void* out, void* out2,
-                            hipStream_t stream, bool after_reduction) {
-  constexpr int kUnroll = 8;
+                            hipStream_t stream) {
+  // 4 loads in flight per lane and 2 workgroups per CU (32 KB per CU) is the best point of the
+  // measured grid {2, 4, 8 loads} x {1..32 workgroups}, alone and right behind the reduction
+  // (bf16 8192^2: 32.6 us against 33.8 with 8 x 2 and 41 with 8 x 8; more in flight is slower)
+  constexpr int kUnroll = 4;
   constexpr size_t kStoreAlign = IN == DT_F32 ? 4 : 8;
   uint8_t* o = static_cast<uint8_t*>(out);
   uint8_t* o2 = static_cast<uint8_t*>(out2);
   const bool fast = aligned(x, 16) && aligned(out, kStoreAlign) && (!PAIR || aligned(out2, kStoreAlign));
   if (fast) {
     const int64_t nvec = numel / InTraits<IN>::kVec, tail = numel % InTraits<IN>::kVec;
-    // the pair cast right behind the reduction finds part of x in the memory-side cache and likes a
-    // larger grid (3 per CU: 61.5 vs 64 us for the step); on its own one workgroup per CU is best (45 vs 50.6 us)
-    int grid = reduction_grid(nvec, kUnroll, !PAIR ? "cast.blocks_per_cu" : after_reduction ? "cast.pair_blocks_per_cu" : "cast.pair_alone_blocks_per_cu");
+    int grid = reduction_grid(nvec, kUnroll, PAIR ? "cast.pair_blocks_per_cu" : "cast.blocks_per_cu");
     cast_kernel<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR, kUnroll><<<grid, kBlock, 0, stream>>>(x, nvec, tail, scale, o, o2);
   } else {
     int grid = reduction_grid(numel, 1, "cast.blocks_per_cu");
@@ -298,8 +299,8 @@ inline int launch_cast_impl(const void* x, int64_t numel, const float* scale, vo
 // other fp8 type with scale[1].
 template <bool PAIR>
 inline int launch_cast(const void* x, int in_dtype, int64_t numel, const float* scale, int out_dtype,
-                       int round_mode, void* out, void* out2, hipStream_t stream, bool after_reduction = false) {
-#define DT_CAST(IN, OUT, RB, RS) return launch_cast_impl<IN, OUT, RB, RS, PAIR>(x, numel, scale, out, out2, stream, after_reduction)
+                       int round_mode, void* out, void* out2, hipStream_t stream) {
+#define DT_CAST(IN, OUT, RB, RS) return launch_cast_impl<IN, OUT, RB, RS, PAIR>(x, numel, scale, out, out2, stream)
   if (in_dtype == DT_F32) {
     if (out_dtype == DT_E4M3FN) DT_CAST(DT_F32, DT_E4M3FN, false, false);
     DT_CAST(DT_F32, DT_E5M2, false, false);
