@@ -27,7 +27,7 @@ Knob g_knobs[] = {
     {"cast.blocks_per_cu", 2},
     {"cast.pair_blocks_per_cu", 2},
     {"mx.blocks_per_cu", 32},
-    {"mx.col_blocks_per_cu", 16},
+    {"mx.col_blocks_per_cu", 32},
     {"mx.dual", 1},
     {"mx.row_band4", 1},
     {"gemm.variant", 0},
