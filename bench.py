@@ -32,7 +32,7 @@ MALL_BYTES = 256 << 20
 # HBM-side bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, each
 # scaled by what the same counter reads for a plain 128 MiB device copy (fetch x1.9996, write
 # x1.0): profiles/dynamic_quant_pair_config2_hbm_traffic.txt
-CAST_PAIR_TRAFFIC_BYTES = 268.69e6
+CAST_PAIR_TRAFFIC_BYTES = 268.57e6
 RESIDENT_PAIR_TRAFFIC_BYTES = 269.38e6  # same method, resident_quant_kernel (one read of x, two fp8 writes)
 
 
