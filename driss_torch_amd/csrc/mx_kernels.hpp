@@ -475,7 +475,9 @@ __device__ __forceinline__ uint32_t other_half_max_pk16(uint32_t v) {  // v: two
   return pk_absmax16(r[0], r[1]);
 }
 
-template <int IN, int OUT, int LAYOUT>
+// WITH_ROWS = false leaves out the row-wise half (data_r / scale_r unused): the transposed column
+// cast on its own.  cols then only has to be a multiple of a lane's kV columns.
+template <int IN, int OUT, int LAYOUT, bool WITH_ROWS = true>
 __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict__ x, uint32_t rows, uint32_t cols,
                                                          uint8_t* __restrict__ data_r, uint8_t* __restrict__ scale_r,
                                                          uint8_t* __restrict__ data_c, uint8_t* __restrict__ scale_c, int cols_first) {
@@ -579,7 +581,7 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
   uint32_t rb[4] = {0u, 0u, 0u, 0u};  // this lane's 16 row-scale bytes, rows in byte order
   uint8_t* drow = data_r + (uint64_t)row0 * cols + col0;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
+  for (int i = 0; i < (WITH_ROWS ? 16 : 0); ++i) {
     uint32_t m = quad_umax(vec_absmax_bits<IN>(v[i]));
     if constexpr (LPB == 8) m = umax(m, dpp<kDppRowHalfMirror>(m));
     const MxScale<OUT> s = mx_scale_from_absbits<OUT>(m);
@@ -597,7 +599,7 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
       }
     }
   }
-  if ((c8 % LPB) == 0)  // inactive lanes hold zero bytes: what the padding of the blocked layout must be
+  if (WITH_ROWS && (c8 % LPB) == 0)  // inactive lanes hold zero bytes: what the padding of the blocked layout must be
     *reinterpret_cast<u32x4*>(rtile + (c8 / LPB) * kDualRows + lrow0) = u32x4{rb[0], rb[1], rb[2], rb[3]};
   __syncthreads();
 
@@ -628,7 +630,7 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
   }
   // ---- row-block scales [rows, cols/32]: kRowBlocks bytes per row of this tile
   const uint32_t KB = cols / 32, kb0 = tc * kRowBlocks;
-  if (tid < kDualRows && trow0 + tid < rows) {
+  if (WITH_ROWS && tid < kDualRows && trow0 + tid < rows) {
     const uint32_t r = trow0 + tid;
 #pragma unroll
     for (int g = 0; g < kRowBlocks / 4; ++g) {

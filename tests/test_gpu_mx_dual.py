@@ -23,7 +23,7 @@ def d(gpu_device):
 def cabi(gpu_device):
     from driss_torch_amd import cabi as c
 
-    keep = {k: c.get_tuning(k) for k in ("mx.dual", "mx.row_band4")}
+    keep = {k: c.get_tuning(k) for k in ("mx.dual", "mx.row_band4", "mx.colt_via_dual")}
     yield c
     for k, v in keep.items():
         c.set_tuning(k, v)
@@ -163,3 +163,24 @@ def test_mx_casts_every_bf16_pattern(d, out_dtype):
             dr, sr, dc, sc = d.mx_fp8_quantize_dual(g, out_dtype)
             assert torch.equal(util.codes(dr), rd) and torch.equal(util.codes(sr), rs.flatten())
             assert torch.equal(util.codes(dc), cd) and torch.equal(util.codes(sc), cs.flatten())
+
+
+@pytest.mark.parametrize("shape", [(32, 8), (64, 36), (128, 100), (160, 264), (992, 1312), (2048, 4096)], ids=lambda s: f"{s[0]}x{s[1]}")
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_transposed_column_cast_both_kernels(d, cabi, shape, in_dtype):
+    """the transposed column cast runs as the one-read kernel without its row half when a lane's 8 (fp32: 4)
+    columns are whole, otherwise (36 and 100 columns of 16-bit data) as the 4-columns-per-lane kernel; with
+    the switch off always as the latter.  Both against the oracle, plain and blocked scales."""
+    x = _wide_range(shape, 33, in_dtype)
+    if shape[0] >= 64:
+        x[40, 3] = float("nan")
+        x[32:64, 5] = 0
+    g = x.cuda()
+    for out_dtype in (E4, E5):
+        cd, cs = co.mx_quantize(x, axis=0, transpose=True, out_dtype=out_dtype)
+        for via_dual in (1, 0):
+            cabi.set_tuning("mx.colt_via_dual", via_dual)
+            data, scale = d.mx_fp8_quantize(g, 32, 0, True, out_dtype)
+            assert torch.equal(util.codes(data), cd) and torch.equal(util.codes(scale), cs.flatten())
+            data, scale = d.mx_fp8_quantize_blocked(g, 0, out_dtype)
+            assert torch.equal(util.codes(data), cd) and torch.equal(util.codes(scale), co.to_blocked(cs))
