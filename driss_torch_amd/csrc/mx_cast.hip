@@ -112,7 +112,7 @@ int launch_dual(const DualArgs& a) {
   const int64_t tiles = ceil_div(a.rows, (int64_t)kDualRows) * ceil_div(a.cols, (int64_t)kTileCols);
   if (tiles > 0x7FFFFFFFll) return kNotTaken;
   mx_dual_kernel<IN, OUT, LAYOUT><<<(unsigned)tiles, kBlock, 0, a.stream>>>(a.x, (uint32_t)a.rows, (uint32_t)a.cols, a.data_r,
-                                                                           a.scale_r, a.data_c, a.scale_c, a.cols <= a.rows ? 1 : 0);
+                                                                           a.scale_r, a.data_c, a.scale_c, a.cols > 2 * a.rows ? 0 : 1);
   return launch_status();
 }
 template <int IN>

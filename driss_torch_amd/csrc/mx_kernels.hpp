@@ -494,8 +494,9 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
   // Tile order.  Along the columns first keeps neighbouring workgroups on the same rows of the
   // input and of the row-wise payload; down the rows first (in runs of 8 tiles per XCD, as in
   // mx_col_t_kernel) keeps them on the same rows of the transposed payload.  Measured, the first
-  // is faster unless the matrix is wider than tall (16384 x 4096 bf16: 54 vs 63 us; 4096 x
-  // 16384: 59 vs 54 us), so the host picks by shape.
+  // is faster unless the matrix is much wider than tall (16384 x 4096 bf16: 50 vs 57 us; 4096 x
+  // 16384: 53 vs 52 us; without the row-wise half the second wins from square on), so the host
+  // picks by shape.
   const uint32_t row_tiles = (rows + kDualRows - 1) / kDualRows;
   uint32_t tr, tc;
   if (cols_first) {
