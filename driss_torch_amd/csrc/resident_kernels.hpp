@@ -279,14 +279,19 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
   if (grid > cus) grid = cus;
   if (grid < 1) grid = 1;
   auto kernel = resident_quant_kernel<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR>;
-  static bool configured = false;  // per instantiation; the attribute is idempotent, a race only repeats the call
-  if (!configured) {
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  if (dev < 0 || dev >= ResidentGate::kMaxDevices) return kResidentNotTaken;
+  // per instantiation and device (a function's attributes live with the device's copy of the code);
+  // the call is idempotent, so a race between threads only repeats it
+  static bool configured[ResidentGate::kMaxDevices] = {};
+  if (!configured[dev]) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)kResLdsBytes) != hipSuccess) {
       (void)hipGetLastError();
       return kResidentNotTaken;
     }
-    configured = true;
+    configured[dev] = true;
   }
   uint8_t* w = static_cast<uint8_t*>(ws);
   uint8_t* o = static_cast<uint8_t*>(out);
@@ -302,9 +307,6 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
     (void)hipGetLastError();
     return kResidentNotTaken;
   }
-  int dev = 0;
-  (void)hipGetDevice(&dev);
-  if (dev < 0 || dev >= ResidentGate::kMaxDevices) return kResidentNotTaken;
   if (gate.used[dev] && gate.last_stream[dev] != stream) {
     // mark the tail of the stream that ran the previous resident kernel and wait for it here
     if (!gate.event[dev] && hipEventCreateWithFlags(&gate.event[dev], hipEventDisableTiming) != hipSuccess) {
