@@ -174,6 +174,25 @@ def test_mx_gemm_both_tile_shapes(d, cabi, variant, size):
         cabi.set_tuning("gemm.variant", 0)
 
 
+def _random_gemm_sizes(seed, n):
+    import random
+
+    rng = random.Random(seed)
+    return [(rng.randint(1, 700), 128 * rng.randint(1, 9), 8 * rng.randint(1, 100)) for _ in range(n)]
+
+
+@pytest.mark.parametrize("variant", [0, 2, 8])
+@pytest.mark.parametrize("size", _random_gemm_sizes(7, 8), ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+def test_mx_gemm_random_sizes(d, cabi, variant, size):
+    """(M, K, N) with M arbitrary, N a multiple of 8 (src/mx_fp8_bf16.cu:187), K a multiple of 128: ragged edge
+    tiles in both directions"""
+    cabi.set_tuning("gemm.variant", variant)
+    try:
+        _check_gemm(d, *size, 900 + size[0], "randn")
+    finally:
+        cabi.set_tuning("gemm.variant", 0)
+
+
 def test_mx_gemm_small_vs_c_oracle_exact_products(d):
     """with power-of-two operands in a narrow exponent range every product and partial sum is
     exact, so the bf16 result must equal the C oracle's float64 reference rounded to bf16, bit
