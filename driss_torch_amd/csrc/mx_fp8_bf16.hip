@@ -89,7 +89,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
 
   // ---- global -> LDS.  Wave w owns groups w*kLoads .. of each panel; lane L fills row L/8,
   // chunk position L%8 of the group, i.e. it fetches logical chunk (L%8) ^ (L/8) of that row.
-  // Rows past the edge re-read the last row; their products are never stored.
+  // Rows past the edge re-read the last row; their products are never stored.  The tile's first
+  // row goes into the 64-bit scalar base, so the 32-bit lane offsets only span the tile's rows
+  // and an operand may be larger than 4 GiB.
+  const uint8_t* const A_tile = A + (int64_t)m0 * lda;
+  const uint8_t* const B_tile = B + (int64_t)n0 * ldb;
   const int lrow = lane >> 3, lchunk = (lane & 7) ^ lrow;
   const uint32_t half_adj = (lchunk & 4) ? 64u : 0u;  // in a half-filled step chunks 4-7 re-read chunks 0-3
   uint32_t offA[kLoadsA], offB[kLoadsB];
@@ -97,13 +101,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   for (int i = 0; i < kLoadsA; ++i) {
     int gr = m0 + (wave * kLoadsA + i) * kGroupRows + lrow;
     gr = gr < M ? gr : M - 1;
-    offA[i] = (uint32_t)((int64_t)gr * lda + lchunk * 16);
+    offA[i] = (uint32_t)((int64_t)(gr - m0) * lda + lchunk * 16);
   }
 #pragma unroll
   for (int i = 0; i < kLoadsB; ++i) {
     int gr = n0 + (wave * kLoadsB + i) * kGroupRows + lrow;
     gr = gr < N ? gr : N - 1;
-    offB[i] = (uint32_t)((int64_t)gr * ldb + lchunk * 16);
+    offB[i] = (uint32_t)((int64_t)(gr - n0) * ldb + lchunk * 16);
   }
   // Scales: KC more wave-wide loads per step.  Even waves bring A chunks, odd waves B chunks:
   // lanes 0-31 the tile's first 128-row chunk, lanes 32-63 the next one (the second chunk of a
@@ -111,10 +115,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // them (duplicates write identical bytes), which keeps the instruction stream free of branches.
   const bool wave_is_b = (wave & 1) != 0;
   const int chunk_max = (wave_is_b ? (N + 127) / 128 : (M + 127) / 128) - 1;
-  int chunk = (wave_is_b ? n0 : m0) / 128 + (lane >> 5);
-  chunk = chunk < chunk_max ? chunk : chunk_max;
-  const uint8_t* sc_base = wave_is_b ? sfb : sfa;
-  const uint32_t sc_off = (uint32_t)((int64_t)chunk * k_chunks * 512 + (lane & 31) * 16);
+  const int chunk0 = (wave_is_b ? n0 : m0) / 128;  // the tile's first chunk row: part of the scalar base
+  const int chunk = chunk0 + (lane >> 5) < chunk_max ? chunk0 + (lane >> 5) : chunk_max;
+  const uint8_t* sc_base = (wave_is_b ? sfb : sfa) + (int64_t)chunk0 * k_chunks * 512;
+  const uint32_t sc_off = (uint32_t)((int64_t)(chunk - chunk0) * k_chunks * 512 + (lane & 31) * 16);
   const int sc_dst = wave_is_b ? kOffSB : kOffSA;
   // load number n of a step: n < kLoadsA -> A group, < kLoadsA+kLoadsB -> B group, else scales
   constexpr int kLoadsPerStep = kLoadsA + kLoadsB + KC;
@@ -131,10 +135,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   auto fetch_one = [&](int n, int ks, uint32_t buf) {
     const uint32_t adj = (FP4 && ks == half_step) ? half_adj : 0u;
     if (n < kLoadsA) {
-      dma16(A + (int64_t)ks * kBK, offA[n] - adj, buf + (wave * kLoadsA + n) * kGroupStride);
+      dma16(A_tile + (int64_t)ks * kBK, offA[n] - adj, buf + (wave * kLoadsA + n) * kGroupStride);
     } else if (n < kLoadsA + kLoadsB) {
       const int i = n - kLoadsA;
-      dma16(B + (int64_t)ks * kBK, offB[i] - adj, buf + kOffB + (wave * kLoadsB + i) * kGroupStride);
+      dma16(B_tile + (int64_t)ks * kBK, offB[i] - adj, buf + kOffB + (wave * kLoadsB + i) * kGroupStride);
     } else {
       const int c = n - kLoadsA - kLoadsB;  // chunk of the step; past the end it re-reads the last one (switched off)
       int kc = ks * KC + c;
@@ -444,6 +448,7 @@ template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4, bool TOUC
 int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N,
                 int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream) {
   const int tiles_m = (int)ceil_div(M, BM), tiles_n = (int)ceil_div(N, BN);
+  if ((int64_t)tiles_m * tiles_n > 0x7FFFFFFFll) return DT_ERR_INVALID_SHAPE;  // one workgroup per tile
   // NST K-steps: panels + scale slots (1 KiB per operand and 128-element chunk of the step)
   size_t lds_bytes = (size_t)NST * (((BM + BN) / kGroupRows) * kGroupStride + 2048 * (FP4 ? 2 : 1));
   const size_t epi_bytes = (size_t)WAVES_M * WAVES_N * (BM / WAVES_M) * ((BN / WAVES_N) * 2 + 16);  // epilogue staging
@@ -476,8 +481,8 @@ int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb
   if (!a || !b || !sfa || !sfb || !out) return DT_ERR_NULL_POINTER;
   if (!aligned(a, 16) || !aligned(b, 16) || lda % 16 != 0 || ldb % 16 != 0) return DT_ERR_MISALIGNED;
   if (!aligned(out, 8) || !aligned(sfa, 4) || !aligned(sfb, 4)) return DT_ERR_MISALIGNED;
-  // per-lane byte offsets into A and B are 32 bits wide
-  if ((M - 1) * lda + k_bytes > 0xFFFFFFFFll || (N - 1) * ldb + k_bytes > 0xFFFFFFFFll) return DT_ERR_INVALID_SHAPE;
+  // per-lane byte offsets are 32 bits wide and span the rows of one tile (at most 256)
+  if (255 * lda + k_bytes > 0xFFFFFFFFll || 255 * ldb + k_bytes > 0xFFFFFFFFll) return DT_ERR_INVALID_SHAPE;
   const uint8_t* A = static_cast<const uint8_t*>(a);
   const uint8_t* B = static_cast<const uint8_t*>(b);
   hipStream_t s = as_hip(stream);

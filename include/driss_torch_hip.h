@@ -174,7 +174,8 @@ DT_API int dt_to_blocked(const uint8_t* scale, int64_t R, int64_t C, uint8_t* ou
  * bytes; sfa / sfb: E8M0 in the blocked layout, dt_blocked_scale_bytes(M, K/32) and
  * (N, K/32) bytes.  K % 128 == 0, lda % 16 == 0, ldb % 16 == 0, a, b 16-byte aligned
  * (:190-195), out 8-byte aligned, N % 4 == 0 and ldo % 4 == 0 (the reference asks N % 8, :187);
- * each operand must span less than 4 GiB ((rows-1)*ld + K bytes).                        */
+ * 256 rows of an operand must span less than 4 GiB (255*ld + K bytes); the operand itself
+ * may be larger.                                                                         */
 DT_API int dt_mx_fp8_bf16(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb,
                           int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, void* out,
                           int64_t ldo, dt_stream_t stream);

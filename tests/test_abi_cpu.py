@@ -68,8 +68,9 @@ def test_host_validation_without_gpu():
     assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 128, 126, 128, 128, 128, fake, 126, None) == 2  # N % 4
     assert L.dt_mx_fp8_bf16(fake + 8, fake, fake, fake, 128, 128, 128, 128, 128, fake, 128, None) == 4
     assert L.dt_mx_fp8_bf16(fake, fake, None, fake, 128, 128, 128, 128, 128, fake, 128, None) == 3
-    # per-lane byte offsets into the operands are 32 bits wide
-    assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 1 << 20, 128, 8192, 8192, 8192, fake, 128, None) == 2
+    # per-lane byte offsets span the 256 rows of a tile and are 32 bits wide
+    assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 512, 128, 8192, 1 << 25, 8192, fake, 128, None) == 2
+    assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 128, 512, 8192, 8192, 1 << 25, fake, 512, None) == 2
     # e2m1 operands: K counts elements, the row strides bytes
     assert L.dt_mx_fp4_bf16(fake, fake, fake, fake, 128, 128, 192, 96, 96, fake, 128, None) == 2  # K % 128
     assert L.dt_mx_fp4_bf16(fake, fake, fake, fake, 128, 128, 256, 64, 128, fake, 128, None) == 2  # lda < K/2
