@@ -42,6 +42,9 @@ SIGNATURES = {
     "dt_to_blocked": (_i32, [_vp, _i64, _i64, _vp, _vp]),
     "dt_mx_fp8_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     "dt_mx_fp4_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
+    "dt_mx_gemm_workspace_bytes": (_sz, []),
+    "dt_mx_fp8_bf16_ws": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "dt_mx_fp4_bf16_ws": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "dt_set_tuning": (_i32, [_cp, _i32]),
     "dt_get_tuning": (_i32, [_cp, C.POINTER(_i32)]),
 }
@@ -96,6 +99,22 @@ def workspace(device=None) -> torch.Tensor:
         ws = torch.empty(lib().dt_workspace_bytes(), dtype=torch.uint8, device=dev)
         _check(lib().dt_workspace_init(ws.data_ptr(), ws.numel(), _stream()), "dt_workspace_init")
         _workspaces[key] = ws
+    return ws
+
+
+_gemm_workspaces = {}
+
+
+def gemm_workspace(device=None) -> torch.Tensor:
+    """A split-K workspace (zeroed once) for the current (device, stream)."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    if dev.index is None:
+        dev = torch.device("cuda", torch.cuda.current_device())
+    key = (dev.index, _stream())
+    ws = _gemm_workspaces.get(key)
+    if ws is None:
+        ws = torch.zeros(lib().dt_mx_gemm_workspace_bytes(), dtype=torch.uint8, device=dev)
+        _gemm_workspaces[key] = ws
     return ws
 
 
@@ -222,21 +241,36 @@ def to_blocked(scale: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def mx_fp8_bf16(a: torch.Tensor, bt: torch.Tensor, sfa: torch.Tensor, sfb: torch.Tensor, out=None) -> torch.Tensor:
-    """a [M,K], bt [N,K] (both K-contiguous), blocked scales -> bf16 [M,N]."""
+def mx_fp8_bf16(a: torch.Tensor, bt: torch.Tensor, sfa: torch.Tensor, sfb: torch.Tensor, out=None,
+                workspace: bool = True) -> torch.Tensor:
+    """a [M,K], bt [N,K] (both K-contiguous), blocked scales -> bf16 [M,N].  ``workspace=False`` calls
+    the entry point without a split-K workspace."""
     M, K = a.shape
     N = bt.shape[0]
     out = torch.empty((M, N), dtype=torch.bfloat16, device=a.device) if out is None else out
-    _check(lib().dt_mx_fp8_bf16(a.data_ptr(), bt.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), M, N, K, a.stride(0),
-                                bt.stride(0), out.data_ptr(), out.stride(0), _stream()), "dt_mx_fp8_bf16")
+    if workspace:
+        ws = gemm_workspace(a.device)
+        _check(lib().dt_mx_fp8_bf16_ws(a.data_ptr(), bt.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), M, N, K, a.stride(0),
+                                       bt.stride(0), out.data_ptr(), out.stride(0), ws.data_ptr(), ws.numel(), _stream()),
+               "dt_mx_fp8_bf16_ws")
+    else:
+        _check(lib().dt_mx_fp8_bf16(a.data_ptr(), bt.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), M, N, K, a.stride(0),
+                                    bt.stride(0), out.data_ptr(), out.stride(0), _stream()), "dt_mx_fp8_bf16")
     return out
 
 
-def mx_fp4_bf16(a: torch.Tensor, bt: torch.Tensor, sfa: torch.Tensor, sfb: torch.Tensor, out=None) -> torch.Tensor:
+def mx_fp4_bf16(a: torch.Tensor, bt: torch.Tensor, sfa: torch.Tensor, sfb: torch.Tensor, out=None,
+                workspace: bool = True) -> torch.Tensor:
     """a [M,K/2], bt [N,K/2] packed e2m1 pairs (both K-contiguous), blocked scales -> bf16 [M,N]."""
     M, Kp = a.shape
     N = bt.shape[0]
     out = torch.empty((M, N), dtype=torch.bfloat16, device=a.device) if out is None else out
-    _check(lib().dt_mx_fp4_bf16(a.data_ptr(), bt.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), M, N, 2 * Kp, a.stride(0),
-                                bt.stride(0), out.data_ptr(), out.stride(0), _stream()), "dt_mx_fp4_bf16")
+    if workspace:
+        ws = gemm_workspace(a.device)
+        _check(lib().dt_mx_fp4_bf16_ws(a.data_ptr(), bt.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), M, N, 2 * Kp, a.stride(0),
+                                       bt.stride(0), out.data_ptr(), out.stride(0), ws.data_ptr(), ws.numel(), _stream()),
+               "dt_mx_fp4_bf16_ws")
+    else:
+        _check(lib().dt_mx_fp4_bf16(a.data_ptr(), bt.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), M, N, 2 * Kp, a.stride(0),
+                                    bt.stride(0), out.data_ptr(), out.stride(0), _stream()), "dt_mx_fp4_bf16")
     return out

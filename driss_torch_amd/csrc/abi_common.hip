@@ -22,6 +22,8 @@ struct Knob {
 //   mx.row_band4: 1 = row-wise MX cast with blocked scales walks 4 rows x 512 elements per wave pass
 //   gemm.variant: 0 = pick the tile by problem size, 1 = 128x128 tiles, 2 = 256x256 tiles,
 //                 7 = 256x256 tiles without the L2 prefetch loads, 8 = 256x256 tiles on 8 waves (e4m3 only)
+//   gemm.split_k: 0 = share K between workgroups when the 128x128 tiling leaves CUs idle (needs the
+//                 workspace of the _ws entry points), 1 = never, n = n workgroups per tile
 Knob g_knobs[] = {
     {"amax.blocks_per_cu", 1},
     {"amax.stream_before_cast", 0},
@@ -33,6 +35,7 @@ Knob g_knobs[] = {
     {"mx.colt_via_dual", 1},
     {"mx.row_band4", 1},
     {"gemm.variant", 0},
+    {"gemm.split_k", 0},
     {"dynamic.resident", 1},
     {"dynamic.resident_min_kib", 0},
     {"dynamic.resident_gap_lo_kib", 12288},

@@ -33,6 +33,10 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 constexpr int kBK = 128;             // K bytes per step = one 16x16x128 MFMA
 constexpr int kGroupRows = 8;        // rows filled by one wave-wide LDS-DMA load
 constexpr int kGroupStride = 1024;   // 8 rows of 128 bytes; the chunk swizzle alone makes fragment reads conflict-free (measured)
+constexpr size_t kSplitTicketBytes = 1024;        // head of the split-K workspace: one counter per 128 x 128 tile
+constexpr size_t kSplitTileBytes = 128 * 128 * 4;  // parked fp32 accumulators of one tile and split
+constexpr int kMaxSplits = 16;      // what gemm.split_k may force
+constexpr int kAutoMaxSplits = 12;  // what the library picks by itself
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
@@ -43,11 +47,24 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 // elements = two MFMAs: bytes 16g.. of the first half feed the first, bytes 64+16g.. the second,
 // which are the same two 16-byte reads a lane makes for e4m3.  Everything else (panels, DMA,
 // swizzle, ring, quadrant schedule, epilogue) is shared; a K-step carries twice the scales.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4, bool TOUCH>
+//
+// SPLIT: the K-steps of a tile are shared between `splits` workgroups (workgroup = tile + split *
+// tiles).  Each parks its fp32 accumulators in `partial`, lane for lane, and takes a ticket of
+// its tile; whoever draws the last ticket adds the parked accumulators in split order (so the sum
+// does not depend on who came last), writes the bf16 tile and puts the ticket counter back to
+// zero.  Nobody waits for anybody.
+// The parked accumulators travel as device-scope relaxed atomics (stores that write through the
+// XCD's L2, loads that miss it): ordinary stores would need a release and an acquire fence around
+// the ticket, i.e. a write-back and an invalidation of the whole L2 that every other workgroup
+// of the XCD is reading its panels through (measured: 1024^3 20.5 us with the fences, 8.8 us
+// without splitting).
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4, bool TOUCH, bool SPLIT>
 __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const uint8_t* __restrict__ sfa,
     const uint8_t* __restrict__ sfb, int M, int N, int K, int64_t lda, int64_t ldb, uint16_t* __restrict__ out,
-    int64_t ldo, int tiles_m, int tiles_n, int wide_stores) {
+    int64_t ldo, int tiles_m, int tiles_n, int wide_stores, int splits, v4f* __restrict__ partial,
+    uint32_t* __restrict__ tickets) {
+  static_assert(!(SPLIT && TOUCH), "the prefetch shares assume that a workgroup walks the whole K");
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
   constexpr int TM = WM / 16, TN = WN / 16;            // MFMA tiles per wave
   constexpr int KC = FP4 ? 2 : 1;                      // 128-element MFMAs (and blocked scale chunks) per K-step
@@ -71,6 +88,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // ids so that neighbours in the tile grid share an L2, then walk tiles in column groups.
   int bid = blockIdx.x;
   const int nb = tiles_m * tiles_n;
+  int split = 0;
+  if constexpr (SPLIT) {
+    split = bid / nb;
+    bid -= split * nb;
+  }
   if (nb % 8 == 0) bid = (bid % 8) * (nb / 8) + bid / 8;
   constexpr int kGroup = 8;  // tile rows per group
   const int group_size = kGroup * tiles_n;
@@ -83,17 +105,27 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // step may be half filled (K % 256 == 128): its second MFMA is then switched off through the
   // scales (see scale_bits) and its loads stay inside the first 64 bytes.
   const int k_bytes = FP4 ? K / 2 : K;
-  const int k_steps = (k_bytes + kBK - 1) / kBK;
+  int k_steps = (k_bytes + kBK - 1) / kBK;
   const int k_chunks = K / 128;                                   // blocked scale chunks per 128 rows
-  const int half_step = (FP4 && (k_bytes % kBK) != 0) ? k_steps - 1 : -1;  // index of a half-filled step
+  int half_step = (FP4 && (k_bytes % kBK) != 0) ? k_steps - 1 : -1;  // index of a half-filled step
+  // SPLIT: this workgroup walks steps ks_begin .. ks_begin + k_steps; from here on steps and scale
+  // chunks count from ks_begin (the host makes sure that every split owns a step)
+  int ks_begin = 0, k_chunks_left = k_chunks;
+  if constexpr (SPLIT) {
+    const int per = (k_steps + splits - 1) / splits;
+    ks_begin = split * per;
+    k_steps = k_steps - ks_begin < per ? k_steps - ks_begin : per;
+    half_step -= ks_begin;
+    k_chunks_left -= ks_begin * KC;
+  }
 
   // ---- global -> LDS.  Wave w owns groups w*kLoads .. of each panel; lane L fills row L/8,
   // chunk position L%8 of the group, i.e. it fetches logical chunk (L%8) ^ (L/8) of that row.
   // Rows past the edge re-read the last row; their products are never stored.  The tile's first
   // row goes into the 64-bit scalar base, so the 32-bit lane offsets only span the tile's rows
   // and an operand may be larger than 4 GiB.
-  const uint8_t* const A_tile = A + (int64_t)m0 * lda;
-  const uint8_t* const B_tile = B + (int64_t)n0 * ldb;
+  const uint8_t* const A_tile = A + (int64_t)m0 * lda + (int64_t)ks_begin * kBK;
+  const uint8_t* const B_tile = B + (int64_t)n0 * ldb + (int64_t)ks_begin * kBK;
   const int lrow = lane >> 3, lchunk = (lane & 7) ^ lrow;
   const uint32_t half_adj = (lchunk & 4) ? 64u : 0u;  // in a half-filled step chunks 4-7 re-read chunks 0-3
   uint32_t offA[kLoadsA], offB[kLoadsB];
@@ -117,7 +149,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   const int chunk_max = (wave_is_b ? (N + 127) / 128 : (M + 127) / 128) - 1;
   const int chunk0 = (wave_is_b ? n0 : m0) / 128;  // the tile's first chunk row: part of the scalar base
   const int chunk = chunk0 + (lane >> 5) < chunk_max ? chunk0 + (lane >> 5) : chunk_max;
-  const uint8_t* sc_base = (wave_is_b ? sfb : sfa) + (int64_t)chunk0 * k_chunks * 512;
+  const uint8_t* sc_base = (wave_is_b ? sfb : sfa) + ((int64_t)chunk0 * k_chunks + (int64_t)ks_begin * KC) * 512;
   const uint32_t sc_off = (uint32_t)((int64_t)(chunk - chunk0) * k_chunks * 512 + (lane & 31) * 16);
   const int sc_dst = wave_is_b ? kOffSB : kOffSA;
   // load number n of a step: n < kLoadsA -> A group, < kLoadsA+kLoadsB -> B group, else scales
@@ -142,7 +174,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     } else {
       const int c = n - kLoadsA - kLoadsB;  // chunk of the step; past the end it re-reads the last one (switched off)
       int kc = ks * KC + c;
-      kc = kc < k_chunks ? kc : k_chunks - 1;
+      kc = kc < k_chunks_left ? kc : k_chunks_left - 1;
       dma16(sc_base + (int64_t)kc * 512, sc_off, buf + sc_dst + c * 1024);
     }
   };
@@ -407,6 +439,70 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
+  if constexpr (SPLIT) {
+    __shared__ uint32_t drawn;
+    const int tile_id = tile_m * tiles_n + tile_n;
+    const size_t per_split = (size_t)nb * (kWaves * TM * TN * kWave);  // accumulators (4 floats each) per split
+    // a wave's 16 x 16 tile is two planes of 64 x 8 bytes (the accumulator's first and second pair
+    // of floats), so that each 8-byte store instruction writes 512 contiguous bytes
+    uint64_t* const mine = reinterpret_cast<uint64_t*>(partial + ((size_t)tile_id * kWaves + wave) * (TM * TN * kWave)) + lane;
+    // 16 x 16 tiles wholly outside the matrix are neither parked nor added (uniform per wave)
+    auto inside = [&](int i, int j) { return m0 + wm * WM + i * 16 < M && n0 + wn * WN + j * 16 < N; };
+    typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+    auto park = [](uint64_t* q, v4f v) {
+      const u64x2 w = __builtin_bit_cast(u64x2, v);
+      __hip_atomic_store(q, w.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(q + kWave, w.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+    auto fetch_parked = [](const uint64_t* q) -> v4f {
+      u64x2 w;
+      w.x = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      w.y = __hip_atomic_load(q + kWave, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return __builtin_bit_cast(v4f, w);
+    };
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        if (inside(i, j)) park(mine + (split * per_split + (i * TN + j) * kWave) * 2, acc[i][j]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the parked values have arrived before the ticket is drawn
+    __syncthreads();
+    if (tid == 0) drawn = __hip_atomic_fetch_add(tickets + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (drawn != (uint32_t)(splits - 1)) return;
+    if (tid == 0) tickets[tile_id] = 0u;  // every split has drawn: ready for the next launch
+    // The loads of kBatch splits first, then the additions in split order: a round trip to memory
+    // per kBatch splits, not one per split and tile.  The workgroup's own share is read back like
+    // the others (the same bits as in its registers), which keeps the loop free of selects; tiles
+    // outside the matrix and splits past the last add zeros.
+    constexpr int kBatch = 4;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int sp0 = 0; sp0 < splits; sp0 += kBatch) {
+      v4f p[kBatch][TM][TN];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            p[u][i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+            if (sp0 + u < splits && inside(i, j))
+              p[u][i][j] = fetch_parked(mine + ((sp0 + u) * per_split + (i * TN + j) * kWave) * 2);
+          }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) acc[i][j] += p[u][i][j];
+    }
+    __syncthreads();  // `drawn` and the epilogue staging share no bytes, but keep the waves together
+  }
+
   // ---- epilogue: fp32 -> bf16 (v_cvt_pk_bf16_f32, round to nearest even) and out through LDS.
   // A lane holds 4 consecutive columns of one row per tile; written straight to memory that is
   // 32-byte pieces of 16 different rows per store.  Instead every wave parks its WM x WN tile
@@ -444,9 +540,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4, bool TOUCH>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4, bool TOUCH, bool SPLIT = false>
 int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N,
-                int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream) {
+                int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream, int splits = 1,
+                void* workspace = nullptr) {
   const int tiles_m = (int)ceil_div(M, BM), tiles_n = (int)ceil_div(N, BN);
   if ((int64_t)tiles_m * tiles_n > 0x7FFFFFFFll) return DT_ERR_INVALID_SHAPE;  // one workgroup per tile
   // NST K-steps: panels + scale slots (1 KiB per operand and 128-element chunk of the step)
@@ -456,22 +553,62 @@ int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const ui
   if (lds_bytes < epi_bytes) lds_bytes = epi_bytes;
   // A grid that fits the chip once should land one workgroup per CU: asking for more than half
   // of the LDS keeps the dispatcher from pairing two workgroups on one CU while others idle.
-  if ((int64_t)tiles_m * tiles_n <= device_facts().cu_count && lds_bytes < 82 * 1024) lds_bytes = 82 * 1024;
-  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST, FP4, TOUCH>;
+  if ((int64_t)tiles_m * tiles_n * splits <= device_facts().cu_count && lds_bytes < 82 * 1024) lds_bytes = 82 * 1024;
+  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST, FP4, TOUCH, SPLIT>;
   if (lds_bytes > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess)
       return DT_ERR_LAUNCH;
   }
-  kernel<<<(unsigned)(tiles_m * tiles_n), WAVES_M * WAVES_N * kWave, lds_bytes, stream>>>(
-      a, b, sfa, sfb, (int)M, (int)N, (int)K, lda, ldb, static_cast<uint16_t*>(out), ldo, tiles_m, tiles_n, (ldo % 8 == 0 && aligned(out, 16)) ? 1 : 0);
+  uint8_t* const ws = static_cast<uint8_t*>(workspace);  // ticket counters, then the parked accumulators
+  kernel<<<(unsigned)(tiles_m * tiles_n * splits), WAVES_M * WAVES_N * kWave, lds_bytes, stream>>>(
+      a, b, sfa, sfb, (int)M, (int)N, (int)K, lda, ldb, static_cast<uint16_t*>(out), ldo, tiles_m, tiles_n,
+      (ldo % 8 == 0 && aligned(out, 16)) ? 1 : 0, splits, ws ? reinterpret_cast<v4f*>(ws + kSplitTicketBytes) : nullptr,
+      reinterpret_cast<uint32_t*>(ws));
   return launch_status();
+}
+
+size_t split_workspace_bytes() { return kSplitTicketBytes + (size_t)device_facts().cu_count * kSplitTileBytes; }
+
+// Split-K factor for the 128 x 128 tiling.  A grid of a third of a workgroup per CU or less leaves
+// most of the chip idle while each workgroup walks the whole K, one K-step per memory latency / 3:
+// share K between as many workgroups per tile as fill the chip once.  What it costs is the last
+// workgroup of a tile reading every share through one CU (about 1 us per share of a full tile),
+// so a share is at least 16 K-steps and two shares are not worth it (measured on MI355X, e4m3,
+// us without -> with: 16 x 8192 x 8192 31 -> 19, 128 x 8192 x 8192 31 -> 24, 1024 x 1024 x 16384
+// 58 -> 34, 512 x 512 x 65536 219 -> 50, 128 x 128 x 16384 56 -> 25; no gain: 256 x 8192 x 8192 with
+// two shares 31.5 -> 32.4, 1024 x 1024 x 4096 with four shares of 8 steps 18.3 -> 19.3).  The knob
+// gemm.split_k forces a factor (1 = never split); whatever is asked for, every split owns a step
+// and the workspace holds all shares.
+int plan_splits(int64_t M, int64_t N, int64_t k_steps, size_t workspace_bytes) {
+  const int64_t tiles = ceil_div(M, 128) * ceil_div(N, 128);
+  if (workspace_bytes <= kSplitTicketBytes || tiles > (int64_t)(kSplitTicketBytes / 4)) return 1;
+  const int64_t room = (int64_t)((workspace_bytes - kSplitTicketBytes) / kSplitTileBytes) / tiles;
+  const int forced = tuning("gemm.split_k");
+  int64_t want;
+  if (forced > 0) {
+    want = forced;
+  } else {
+    const int cus = device_facts().cu_count;
+    if (tiles * 3 > cus) return 1;
+    want = cus / tiles;
+    if (want > k_steps / 16) want = k_steps / 16;
+    if (want > kAutoMaxSplits) want = kAutoMaxSplits;
+    if (want < 3) return 1;
+  }
+  if (want > kMaxSplits) want = kMaxSplits;
+  if (want > room) want = room;
+  if (want > k_steps) want = k_steps;
+  if (want < 2) return 1;
+  const int64_t per = ceil_div(k_steps, want);
+  return (int)ceil_div(k_steps, per);
 }
 
 // Shared argument checks and tile choice.  K counts elements, lda/ldb bytes.
 template <bool FP4>
 int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N, int64_t K,
-            int64_t lda, int64_t ldb, void* out, int64_t ldo, dt_stream_t stream) {
+            int64_t lda, int64_t ldb, void* out, int64_t ldo, void* workspace, size_t workspace_bytes,
+            dt_stream_t stream) {
   if (M < 0 || N < 0 || K < 0) return DT_ERR_INVALID_SHAPE;
   if (M == 0 || N == 0) return DT_OK;
   if (K == 0 || K % 128 != 0) return DT_ERR_INVALID_SHAPE;  // one scaled MFMA covers 128 elements
@@ -481,6 +618,7 @@ int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb
   if (!a || !b || !sfa || !sfb || !out) return DT_ERR_NULL_POINTER;
   if (!aligned(a, 16) || !aligned(b, 16) || lda % 16 != 0 || ldb % 16 != 0) return DT_ERR_MISALIGNED;
   if (!aligned(out, 8) || !aligned(sfa, 4) || !aligned(sfb, 4)) return DT_ERR_MISALIGNED;
+  if (workspace && !aligned(workspace, 256)) return DT_ERR_MISALIGNED;
   // per-lane byte offsets are 32 bits wide and span the rows of one tile (at most 256)
   if (255 * lda + k_bytes > 0xFFFFFFFFll || 255 * ldb + k_bytes > 0xFFFFFFFFll) return DT_ERR_INVALID_SHAPE;
   const uint8_t* A = static_cast<const uint8_t*>(a);
@@ -497,6 +635,9 @@ int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb
   }
   if (big && variant == 7) return launch_gemm<256, 256, 2, 2, 2, FP4, false>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
   if (big) return launch_gemm<256, 256, 2, 2, 2, FP4, true>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  const int splits = workspace ? plan_splits(M, N, ceil_div(k_bytes, (int64_t)kBK), workspace_bytes) : 1;
+  if (splits > 1)
+    return launch_gemm<128, 128, 2, 2, 4, FP4, false, true>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s, splits, workspace);
   return launch_gemm<128, 128, 2, 2, 4, FP4, false>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
 }
 
@@ -505,11 +646,25 @@ int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb
 extern "C" int dt_mx_fp8_bf16(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M,
                               int64_t N, int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo,
                               dt_stream_t stream) {
-  return dt::mx_gemm<false>(a, b, sfa, sfb, M, N, K, lda, ldb, out, ldo, stream);
+  return dt::mx_gemm<false>(a, b, sfa, sfb, M, N, K, lda, ldb, out, ldo, nullptr, 0, stream);
 }
 
 extern "C" int dt_mx_fp4_bf16(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M,
                               int64_t N, int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo,
                               dt_stream_t stream) {
-  return dt::mx_gemm<true>(a, b, sfa, sfb, M, N, K, lda, ldb, out, ldo, stream);
+  return dt::mx_gemm<true>(a, b, sfa, sfb, M, N, K, lda, ldb, out, ldo, nullptr, 0, stream);
+}
+
+extern "C" size_t dt_mx_gemm_workspace_bytes(void) { return dt::split_workspace_bytes(); }
+
+extern "C" int dt_mx_fp8_bf16_ws(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M,
+                                 int64_t N, int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo,
+                                 void* workspace, size_t workspace_bytes, dt_stream_t stream) {
+  return dt::mx_gemm<false>(a, b, sfa, sfb, M, N, K, lda, ldb, out, ldo, workspace, workspace_bytes, stream);
+}
+
+extern "C" int dt_mx_fp4_bf16_ws(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M,
+                                 int64_t N, int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo,
+                                 void* workspace, size_t workspace_bytes, dt_stream_t stream) {
+  return dt::mx_gemm<true>(a, b, sfa, sfb, M, N, K, lda, ldb, out, ldo, workspace, workspace_bytes, stream);
 }

@@ -70,6 +70,21 @@ Tensor& workspace_for(const Tensor& like, dt_stream_t stream) {
   return it->second;
 }
 
+// The same for the GEMM's split-K workspace (ticket counters that the kernel leaves zero, and
+// parked accumulators).
+Tensor& gemm_workspace_for(const Tensor& like, dt_stream_t stream) {
+  static std::mutex mu;
+  static auto* cache = new std::map<std::pair<int, void*>, Tensor>();
+  std::lock_guard<std::mutex> lock(mu);
+  auto key = std::make_pair((int)like.get_device(), (void*)stream);
+  auto it = cache->find(key);
+  if (it == cache->end()) {
+    Tensor ws = at::zeros({(int64_t)dt_mx_gemm_workspace_bytes()}, like.options().dtype(at::kByte));
+    it = cache->emplace(key, ws).first;
+  }
+  return it->second;
+}
+
 void check_hp_input(const Tensor& input) {
   TORCH_CHECK(input.is_cuda(), "Input tensor must be on the GPU");
   TORCH_CHECK(input.scalar_type() == at::kBFloat16 || input.scalar_type() == at::kFloat,
@@ -313,9 +328,10 @@ Tensor mx_fp8_bf16(Tensor a, Tensor b, Tensor a_scale, Tensor b_scale) {
   Tensor out = at::empty({M, N}, a.options().dtype(at::kBFloat16));
   if (M == 0 || N == 0) return out;
   const int64_t lda = M > 1 ? a.stride(0) : K, ldb = N > 1 ? b.stride(1) : K;
-  check_status(dt_mx_fp8_bf16(a.data_ptr(), b.data_ptr(), static_cast<const uint8_t*>(a_scale.data_ptr()),
-                              static_cast<const uint8_t*>(b_scale.data_ptr()), M, N, K, lda, ldb, out.data_ptr(), N,
-                              ctx.stream),
+  Tensor& ws = gemm_workspace_for(a, ctx.stream);
+  check_status(dt_mx_fp8_bf16_ws(a.data_ptr(), b.data_ptr(), static_cast<const uint8_t*>(a_scale.data_ptr()),
+                                 static_cast<const uint8_t*>(b_scale.data_ptr()), M, N, K, lda, ldb, out.data_ptr(), N,
+                                 ws.data_ptr(), ws.numel(), ctx.stream),
                "mx_fp8_bf16");
   return out;
 }
@@ -356,9 +372,10 @@ Tensor mx_fp4_bf16(Tensor a, Tensor b, Tensor a_scale, Tensor b_scale) {
   Tensor out = at::empty({M, N}, a.options().dtype(at::kBFloat16));
   if (M == 0 || N == 0) return out;
   const int64_t lda = M > 1 ? a.stride(0) : Kp, ldb = N > 1 ? b.stride(1) : Kp;
-  check_status(dt_mx_fp4_bf16(a.data_ptr(), b.data_ptr(), static_cast<const uint8_t*>(a_scale.data_ptr()),
-                              static_cast<const uint8_t*>(b_scale.data_ptr()), M, N, K, lda, ldb, out.data_ptr(), N,
-                              ctx.stream),
+  Tensor& ws = gemm_workspace_for(a, ctx.stream);
+  check_status(dt_mx_fp4_bf16_ws(a.data_ptr(), b.data_ptr(), static_cast<const uint8_t*>(a_scale.data_ptr()),
+                                 static_cast<const uint8_t*>(b_scale.data_ptr()), M, N, K, lda, ldb, out.data_ptr(), N,
+                                 ws.data_ptr(), ws.numel(), ctx.stream),
                "mx_fp4_bf16");
   return out;
 }

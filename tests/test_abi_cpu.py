@@ -71,6 +71,12 @@ def test_host_validation_without_gpu():
     # per-lane byte offsets span the 256 rows of a tile and are 32 bits wide
     assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 512, 128, 8192, 1 << 25, 8192, fake, 128, None) == 2
     assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 128, 512, 8192, 8192, 1 << 25, fake, 512, None) == 2
+    # the entry points with a split-K workspace: same checks, plus the workspace's alignment
+    assert L.dt_mx_gemm_workspace_bytes() >= 1024 + 128 * 128 * 4
+    assert L.dt_mx_fp8_bf16_ws(fake, fake, fake, fake, 128, 128, 96, 96, 96, fake, 128, fake, 1 << 20, None) == 2
+    assert L.dt_mx_fp8_bf16_ws(fake, fake, fake, fake, 128, 128, 128, 128, 128, fake, 128, fake + 16, 1 << 20, None) == 4
+    assert L.dt_mx_fp4_bf16_ws(fake, fake, fake, fake, 128, 128, 256, 128, 128, fake, 128, fake + 16, 1 << 20, None) == 4
+    assert L.dt_mx_fp8_bf16_ws(fake, fake, fake, fake, 0, 128, 128, 128, 128, fake, 128, None, 0, None) == 0
     # e2m1 operands: K counts elements, the row strides bytes
     assert L.dt_mx_fp4_bf16(fake, fake, fake, fake, 128, 128, 192, 96, 96, fake, 128, None) == 2  # K % 128
     assert L.dt_mx_fp4_bf16(fake, fake, fake, fake, 128, 128, 256, 64, 128, fake, 128, None) == 2  # lda < K/2

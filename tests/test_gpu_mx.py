@@ -193,6 +193,47 @@ def test_mx_gemm_random_sizes(d, cabi, variant, size):
         cabi.set_tuning("gemm.variant", 0)
 
 
+@pytest.mark.parametrize("splits", [0, 2, 3, 5, 16])
+@pytest.mark.parametrize("size", [(16, 2048, 256), (133, 1664, 264), (300, 1024, 136), (1, 640, 8), (64, 8192, 512)],
+                         ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+def test_mx_gemm_split_k(d, cabi, splits, size):
+    """K shared between several workgroups per tile (forced factors, and the library's own choice):
+    same tolerance as the plain kernel, the same bits on every call (the sum runs in split order
+    whoever finishes last, and the ticket counters come back to zero), uneven shares of K-steps."""
+    cabi.set_tuning("gemm.split_k", splits)
+    try:
+        out, _ = _check_gemm(d, *size, 1100 + size[0], "randn")
+        for _ in range(3):
+            again, _ = _check_gemm(d, *size, 1100 + size[0], "randn")
+            assert torch.equal(again, out)
+    finally:
+        cabi.set_tuning("gemm.split_k", 0)
+
+
+def test_mx_gemm_split_k_workspace_rules(d, cabi):
+    M, K, N = 32, 8192, 256  # 64 K-steps on 2 tiles: the library splits by itself
+    a_data, a_sc, b_data, b_sc = _operands(d, M, K, N, 1200, "randn")
+    sa, sb = d.to_blocked(a_sc), d.to_blocked(b_sc)
+    with_ws = cabi.mx_fp8_bf16(a_data, b_data, sa, sb)
+    without = cabi.mx_fp8_bf16(a_data, b_data, sa, sb, workspace=False)
+    ref = eager.mx_dequant(a_data.cpu(), util.codes(a_sc)).double() @ eager.mx_dequant(b_data.cpu(), util.codes(b_sc)).double().T
+    for got in (with_ws, without):
+        assert eager.compute_error(ref, got.cpu().double()).item() > 50
+    L = cabi.lib()
+    out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    ws = torch.zeros(L.dt_mx_gemm_workspace_bytes() + 256, dtype=torch.uint8, device="cuda")
+    args = (a_data.data_ptr(), b_data.data_ptr(), sa.data_ptr(), sb.data_ptr(), M, N, K, K, K, out.data_ptr(), N)
+    assert L.dt_mx_fp8_bf16_ws(*args, ws.data_ptr() + 8, ws.numel() - 8, None) == 4  # misaligned workspace
+    # a workspace too small for any split: the product is computed without one
+    assert L.dt_mx_fp8_bf16_ws(*args, ws.data_ptr(), 1024, None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, without)
+    assert L.dt_mx_fp8_bf16_ws(*args, ws.data_ptr(), ws.numel() - 256, None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, with_ws)
+    assert int(ws[:1024].view(torch.int32).abs().sum().item()) == 0  # tickets are back at zero
+
+
 def test_mx_gemm_small_vs_c_oracle_exact_products(d):
     """with power-of-two operands in a narrow exponent range every product and partial sum is
     exact, so the bf16 result must equal the C oracle's float64 reference rounded to bf16, bit

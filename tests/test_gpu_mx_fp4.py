@@ -74,6 +74,20 @@ def test_mx_fp4_gemm_both_tile_shapes(d, cabi, variant, size):
         cabi.set_tuning("gemm.variant", 0)
 
 
+@pytest.mark.parametrize("splits", [0, 2, 3, 4, 16])
+@pytest.mark.parametrize("size", [(16, 2048, 256), (133, 1408, 264), (40, 16512, 136)], ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+def test_mx_fp4_gemm_split_k(d, cabi, splits, size):
+    """K shared between workgroups, including a K whose last 256-element step is half filled
+    (1408 = 5.5 steps, 16512 = 64.5, which the library splits by itself): the half step belongs to the last split only."""
+    cabi.set_tuning("gemm.split_k", splits)
+    try:
+        out = _check(d, *size, 1300 + size[0], "randn")
+        for _ in range(3):
+            assert torch.equal(_check(d, *size, 1300 + size[0], "randn"), out)
+    finally:
+        cabi.set_tuning("gemm.split_k", 0)
+
+
 def test_mx_fp4_gemm_bit_exact_when_sums_fit_fp32(d):
     """sparse operands and a narrow scale range: every product and every partial sum is a multiple
     of 2^-6 below 2^12, exact in fp32 in any order, so the result must equal the C oracle's float64
