@@ -19,6 +19,7 @@
 // The MFMA is issued with B as the row operand, so a lane's four accumulators are four
 // consecutive columns of one output row; the epilogue converts to bf16 and goes through LDS so
 // that the stores are whole 256-byte row segments (direct 8-byte stores cost 12% of the run).
+#include <atomic>
 #include <type_traits>
 
 #include "dt_device.hpp"
@@ -556,9 +557,17 @@ int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const ui
   if ((int64_t)tiles_m * tiles_n * splits <= device_facts().cu_count && lds_bytes < 82 * 1024) lds_bytes = 82 * 1024;
   auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST, FP4, TOUCH, SPLIT>;
   if (lds_bytes > 64 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds_bytes) != hipSuccess)
-      return DT_ERR_LAUNCH;
+    // once per instantiation and device, with the largest size asked for so far (a host call per launch otherwise)
+    static std::atomic<int> allowed[16];
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    const bool tracked = dev >= 0 && dev < 16;
+    if (!tracked || allowed[dev].load(std::memory_order_relaxed) < (int)lds_bytes) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds_bytes) != hipSuccess)
+        return DT_ERR_LAUNCH;
+      if (tracked) allowed[dev].store((int)lds_bytes, std::memory_order_relaxed);
+    }
   }
   uint8_t* const ws = static_cast<uint8_t*>(workspace);  // ticket counters, then the parked accumulators
   kernel<<<(unsigned)(tiles_m * tiles_n * splits), WAVES_M * WAVES_N * kWave, lds_bytes, stream>>>(

@@ -97,7 +97,11 @@ def test_ops_replay_from_a_captured_graph(d):
     def run(x, w):
         a, sa = d.mx_fp8_quantize_blocked(x)
         b, sb = d.mx_fp8_quantize_blocked(w)
-        return (d.amax(x), d.saturated_cast(x, scale, E4), d.dynamic_scaled_quant(x, E5),
+        # the same bytes as one tile with 64 K-steps: the GEMM shares K between workgroups (ticket counters
+        # that every replay must find at zero)
+        a2, sa2 = d.mx_fp8_quantize_blocked(x.view(64, 8192))
+        b2, sb2 = d.mx_fp8_quantize_blocked(w.view(32, 8192))
+        return (d.mx_fp8_bf16(a2, b2.t(), sa2, sb2), d.amax(x), d.saturated_cast(x, scale, E4), d.dynamic_scaled_quant(x, E5),
                 d.dynamic_scaled_quant_pair(x), d.dynamic_scaled_quant_rowwise(x, E4), d.mx_fp8_quantize(x),
                 d.mx_fp8_quantize(x, 32, 0, True), d.mx_fp8_quantize_dual(x, E4, True), d.mx_fp8_bf16(a, b.t(), sa, sb))
 
