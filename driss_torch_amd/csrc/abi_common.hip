@@ -22,6 +22,8 @@ struct Knob {
 //   mx.row_band4: 1 = row-wise MX cast with blocked scales walks 4 rows x 512 elements per wave pass
 //   gemm.variant: 0 = pick the tile by problem size, 1 = 128x128 tiles, 2 = 256x256 tiles,
 //                 7 = 256x256 tiles without the L2 prefetch loads, 8 = 256x256 tiles on 8 waves (e4m3 only)
+//   gemm.tail_quads: 1 = tiles left over after whole rounds of 256x256 tiles run as 128x128 quadrants
+//                 when those fit the chip at once, 0 = never, 2 = always
 //   gemm.split_k: 0 = share K between workgroups when the 128x128 tiling leaves CUs idle (needs the
 //                 workspace of the _ws entry points), 1 = never, n = n workgroups per tile
 Knob g_knobs[] = {
@@ -36,6 +38,7 @@ Knob g_knobs[] = {
     {"mx.row_band4", 1},
     {"gemm.variant", 0},
     {"gemm.split_k", 0},
+    {"gemm.tail_quads", 1},
     {"dynamic.resident", 1},
     {"dynamic.resident_min_kib", 0},
     {"dynamic.resident_gap_lo_kib", 12288},

@@ -59,13 +59,20 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 // the ticket, i.e. a write-back and an invalidation of the whole L2 that every other workgroup
 // of the XCD is reading its panels through (measured: 1024^3 20.5 us with the fences, 8.8 us
 // without splitting).
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4, bool TOUCH, bool SPLIT>
+//
+// MODE kQuads: the workgroup computes one 128 x 128 quadrant of a 256 x 256 tile, for the tiles that
+// the 256 x 256 kernel leaves over when its grid is cut to whole rounds of the chip (tiles_m,
+// tiles_n and first_block then describe the 256 x 256 tiling).
+enum GemmMode { kPlain = 0, kSplitK = 1, kQuads = 2 };
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4, bool TOUCH, int MODE>
 __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const uint8_t* __restrict__ sfa,
     const uint8_t* __restrict__ sfb, int M, int N, int K, int64_t lda, int64_t ldb, uint16_t* __restrict__ out,
     int64_t ldo, int tiles_m, int tiles_n, int wide_stores, int splits, v4f* __restrict__ partial,
-    uint32_t* __restrict__ tickets) {
+    uint32_t* __restrict__ tickets, int first_block) {
+  constexpr bool SPLIT = MODE == kSplitK;
   static_assert(!(SPLIT && TOUCH), "the prefetch shares assume that a workgroup walks the whole K");
+  static_assert(MODE != kQuads || (BM == 128 && BN == 128), "quadrants of a 256 x 256 tile");
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
   constexpr int TM = WM / 16, TN = WN / 16;            // MFMA tiles per wave
   constexpr int KC = FP4 ? 2 : 1;                      // 128-element MFMAs (and blocked scale chunks) per K-step
@@ -89,10 +96,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // ids so that neighbours in the tile grid share an L2, then walk tiles in column groups.
   int bid = blockIdx.x;
   const int nb = tiles_m * tiles_n;
-  int split = 0;
+  int split = 0, quad = 0;
   if constexpr (SPLIT) {
     split = bid / nb;
     bid -= split * nb;
+  }
+  if constexpr (MODE == kQuads) {
+    // workgroup 8 * (4 g + quad) + x: quadrant `quad` of tile first_block + 8 g + x, so that a tile's
+    // four quadrants run on one XCD (x) and first_block (a multiple of 8) continues the big kernel's runs
+    const int t = bid >> 3;
+    quad = t & 3;
+    bid = first_block + 8 * (t >> 2) + (bid & 7);
+    if (bid >= nb) return;  // the grid is rounded up to whole groups of 8 tiles
   }
   if (nb % 8 == 0) bid = (bid % 8) * (nb / 8) + bid / 8;
   constexpr int kGroup = 8;  // tile rows per group
@@ -101,7 +116,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   const int gm = (tiles_m - first_m) < kGroup ? (tiles_m - first_m) : kGroup;
   const int tile_m = first_m + (bid % group_size) % gm;
   const int tile_n = (bid % group_size) / gm;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int m0 = MODE == kQuads ? tile_m * 256 + (quad >> 1) * 128 : tile_m * BM;
+  const int n0 = MODE == kQuads ? tile_n * 256 + (quad & 1) * 128 : tile_n * BN;
+  if constexpr (MODE == kQuads) {
+    if (m0 >= M || n0 >= N) return;  // quadrant outside the matrix (the whole workgroup leaves)
+  }
   // K counts elements; a row holds k_bytes bytes, a K-step is 128 of them.  With FP4 the last
   // step may be half filled (K % 256 == 128): its second MFMA is then switched off through the
   // scales (see scale_bits) and its loads stay inside the first 64 bytes.
@@ -541,11 +560,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4, bool TOUCH, bool SPLIT = false>
+// blocks > 0: launch only that many workgroups (the first `blocks` of the tiling, or with kQuads the
+// quadrants of `blocks` 256 x 256 tiles from tile number first_block on)
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4, bool TOUCH, int MODE = kPlain>
 int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N,
                 int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream, int splits = 1,
-                void* workspace = nullptr) {
-  const int tiles_m = (int)ceil_div(M, BM), tiles_n = (int)ceil_div(N, BN);
+                void* workspace = nullptr, int64_t blocks = 0, int first_block = 0) {
+  constexpr int kTileM = MODE == kQuads ? 256 : BM, kTileN = MODE == kQuads ? 256 : BN;
+  const int tiles_m = (int)ceil_div(M, kTileM), tiles_n = (int)ceil_div(N, kTileN);
   if ((int64_t)tiles_m * tiles_n > 0x7FFFFFFFll) return DT_ERR_INVALID_SHAPE;  // one workgroup per tile
   // NST K-steps: panels + scale slots (1 KiB per operand and 128-element chunk of the step)
   size_t lds_bytes = (size_t)NST * (((BM + BN) / kGroupRows) * kGroupStride + 2048 * (FP4 ? 2 : 1));
@@ -555,7 +577,7 @@ int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const ui
   // A grid that fits the chip once should land one workgroup per CU: asking for more than half
   // of the LDS keeps the dispatcher from pairing two workgroups on one CU while others idle.
   if ((int64_t)tiles_m * tiles_n * splits <= device_facts().cu_count && lds_bytes < 82 * 1024) lds_bytes = 82 * 1024;
-  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST, FP4, TOUCH, SPLIT>;
+  auto kernel = mx_gemm_kernel<BM, BN, WAVES_M, WAVES_N, NST, FP4, TOUCH, MODE>;
   if (lds_bytes > 64 * 1024) {
     // once per instantiation and device, with the largest size asked for so far (a host call per launch otherwise)
     static std::atomic<int> allowed[16];
@@ -570,10 +592,12 @@ int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const ui
     }
   }
   uint8_t* const ws = static_cast<uint8_t*>(workspace);  // ticket counters, then the parked accumulators
-  kernel<<<(unsigned)(tiles_m * tiles_n * splits), WAVES_M * WAVES_N * kWave, lds_bytes, stream>>>(
+  int64_t grid = (int64_t)tiles_m * tiles_n * splits;
+  if (blocks > 0) grid = MODE == kQuads ? 32 * ceil_div(blocks, (int64_t)8) : blocks;
+  kernel<<<(unsigned)grid, WAVES_M * WAVES_N * kWave, lds_bytes, stream>>>(
       a, b, sfa, sfb, (int)M, (int)N, (int)K, lda, ldb, static_cast<uint16_t*>(out), ldo, tiles_m, tiles_n,
       (ldo % 8 == 0 && aligned(out, 16)) ? 1 : 0, splits, ws ? reinterpret_cast<v4f*>(ws + kSplitTicketBytes) : nullptr,
-      reinterpret_cast<uint32_t*>(ws));
+      reinterpret_cast<uint32_t*>(ws), first_block);
   return launch_status();
 }
 
@@ -643,10 +667,29 @@ int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb
     if (variant == 8) return launch_gemm<256, 256, 2, 4, 2, false, true>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
   }
   if (big && variant == 7) return launch_gemm<256, 256, 2, 2, 2, FP4, false>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
-  if (big) return launch_gemm<256, 256, 2, 2, 2, FP4, true>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  if (big) {
+    // Whole rounds of the chip on 256 x 256 tiles; what is left over would keep the chip for another
+    // full round however few tiles it is.  When its quadrants fit the chip at once it runs as
+    // 128 x 128 quadrants instead: one round of those takes 0.5-0.6 of a round of tiles (measured on
+    // MI355X, e4m3, us: 4096 x 5120 x 4096, 256 + 64 tiles, 97 -> 77; 4352^2 x 4096, 256 + 33, 97 -> 78;
+    // 4096 x 4352 x 8192, 256 + 16, 177 -> 134; 6144^3, 512 + 64, 216 -> 186; 8448 x 8192^2, 1024 + 32,
+    // 473 -> 436), two rounds of quadrants take as long as the round of tiles (4096 x 6144 x 4096,
+    // 256 + 128: 97 -> 96).  The results are the same bits either way.
+    const int cus = device_facts().cu_count;
+    const int64_t rounds = tiles256 / cus, left = tiles256 % cus;
+    const int tail = tuning("gemm.tail_quads");
+    if (variant == 0 && tail != 0 && rounds >= 1 && left > 0 && cus % 8 == 0 && (tail == 2 || 4 * left <= cus)) {
+      const int st = launch_gemm<256, 256, 2, 2, 2, FP4, true>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s, 1, nullptr,
+                                                                rounds * cus);
+      if (st != DT_OK) return st;
+      return launch_gemm<128, 128, 2, 2, 4, FP4, false, kQuads>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s, 1, nullptr,
+                                                                left, (int)(rounds * cus));
+    }
+    return launch_gemm<256, 256, 2, 2, 2, FP4, true>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  }
   const int splits = workspace ? plan_splits(M, N, ceil_div(k_bytes, (int64_t)kBK), workspace_bytes) : 1;
   if (splits > 1)
-    return launch_gemm<128, 128, 2, 2, 4, FP4, false, true>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s, splits, workspace);
+    return launch_gemm<128, 128, 2, 2, 4, FP4, false, kSplitK>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s, splits, workspace);
   return launch_gemm<128, 128, 2, 2, 4, FP4, false>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
 }
 

@@ -210,6 +210,25 @@ def test_mx_gemm_split_k(d, cabi, splits, size):
         cabi.set_tuning("gemm.split_k", 0)
 
 
+@pytest.mark.parametrize("size", [(4352, 256, 4096), (4100, 256, 4360), (4352, 384, 4352), (8200, 128, 4104)],
+                         ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+def test_mx_gemm_leftover_tiles_as_quadrants(d, cabi, size):
+    """more 256 x 256 tiles than CUs: whole rounds on the big kernel, the tiles left over as 128 x 128
+    quadrants (forced here, whatever the estimate says): every entry written once and right, with
+    tile counts that are and are not multiples of 8 and ragged edges in both directions"""
+    cabi.set_tuning("gemm.tail_quads", 2)
+    try:
+        out, _ = _check_gemm(d, *size, 1400 + size[0], "randn")
+    finally:
+        cabi.set_tuning("gemm.tail_quads", 1)
+    cabi.set_tuning("gemm.tail_quads", 0)
+    try:
+        plain, _ = _check_gemm(d, *size, 1400 + size[0], "randn")
+    finally:
+        cabi.set_tuning("gemm.tail_quads", 1)
+    assert torch.equal(out, plain)  # same K order per entry in both kernels: the same bits
+
+
 def test_mx_gemm_split_k_workspace_rules(d, cabi):
     M, K, N = 32, 8192, 256  # 64 K-steps on 2 tiles: the library splits by itself
     a_data, a_sc, b_data, b_sc = _operands(d, M, K, N, 1200, "randn")
