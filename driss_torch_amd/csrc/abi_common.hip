@@ -23,7 +23,8 @@ struct Knob {
 //   gemm.variant: 0 = pick the tile by problem size, 1 = 128x128 tiles, 2 = 256x256 tiles,
 //                 7 = 256x256 tiles without the L2 prefetch loads, 8 = 256x256 tiles on 8 waves (e4m3 only)
 //   gemm.tail_quads: 1 = tiles left over after whole rounds of 256x256 tiles run as 128x128 quadrants
-//                 when those fit the chip at once, 0 = never, 2 = always
+//                 or 256x128 halves when those fit the chip at once, 0 = never, 2 = always as
+//                 quadrants, 3 = always as halves
 //   gemm.split_k: 0 = share K between workgroups when the 128x128 tiling leaves CUs idle (needs the
 //                 workspace of the _ws entry points), 1 = never, n = n workgroups per tile
 Knob g_knobs[] = {

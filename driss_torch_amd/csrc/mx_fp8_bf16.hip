@@ -63,7 +63,8 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 // MODE kQuads: the workgroup computes one 128 x 128 quadrant of a 256 x 256 tile, for the tiles that
 // the 256 x 256 kernel leaves over when its grid is cut to whole rounds of the chip (tiles_m,
 // tiles_n and first_block then describe the 256 x 256 tiling).
-enum GemmMode { kPlain = 0, kSplitK = 1, kQuads = 2 };
+// MODE kHalves: the same with the 256 x 128 halves of a tile.
+enum GemmMode { kPlain = 0, kSplitK = 1, kQuads = 2, kHalves = 3 };
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4, bool TOUCH, int MODE>
 __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const uint8_t* __restrict__ sfa,
@@ -73,6 +74,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   constexpr bool SPLIT = MODE == kSplitK;
   static_assert(!(SPLIT && TOUCH), "the prefetch shares assume that a workgroup walks the whole K");
   static_assert(MODE != kQuads || (BM == 128 && BN == 128), "quadrants of a 256 x 256 tile");
+  static_assert(MODE != kHalves || (BM == 256 && BN == 128), "halves of a 256 x 256 tile");
+  constexpr bool PARTS = MODE == kQuads || MODE == kHalves;
+  constexpr int kParts = MODE == kQuads ? 4 : 2;  // workgroups per 256 x 256 tile
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
   constexpr int TM = WM / 16, TN = WN / 16;            // MFMA tiles per wave
   constexpr int KC = FP4 ? 2 : 1;                      // 128-element MFMAs (and blocked scale chunks) per K-step
@@ -101,12 +105,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     split = bid / nb;
     bid -= split * nb;
   }
-  if constexpr (MODE == kQuads) {
-    // workgroup 8 * (4 g + quad) + x: quadrant `quad` of tile first_block + 8 g + x, so that a tile's
-    // four quadrants run on one XCD (x) and first_block (a multiple of 8) continues the big kernel's runs
+  if constexpr (PARTS) {
+    // workgroup 8 * (kParts * g + part) + x: part `part` of tile first_block + 8 g + x, so that a tile's
+    // parts run on one XCD (x) and first_block (a multiple of 8) continues the big kernel's runs
     const int t = bid >> 3;
-    quad = t & 3;
-    bid = first_block + 8 * (t >> 2) + (bid & 7);
+    quad = t % kParts;
+    bid = first_block + 8 * (t / kParts) + (bid & 7);
     if (bid >= nb) return;  // the grid is rounded up to whole groups of 8 tiles
   }
   if (nb % 8 == 0) bid = (bid % 8) * (nb / 8) + bid / 8;
@@ -117,8 +121,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   const int tile_m = first_m + (bid % group_size) % gm;
   const int tile_n = (bid % group_size) / gm;
   const int m0 = MODE == kQuads ? tile_m * 256 + (quad >> 1) * 128 : tile_m * BM;
-  const int n0 = MODE == kQuads ? tile_n * 256 + (quad & 1) * 128 : tile_n * BN;
-  if constexpr (MODE == kQuads) {
+  const int n0 = PARTS ? tile_n * 256 + (quad & 1) * 128 : tile_n * BN;
+  if constexpr (PARTS) {
     if (m0 >= M || n0 >= N) return;  // quadrant outside the matrix (the whole workgroup leaves)
   }
   // K counts elements; a row holds k_bytes bytes, a K-step is 128 of them.  With FP4 the last
@@ -566,7 +570,8 @@ template <int BM, int BN, int WAVES_M, int WAVES_N, int NST, bool FP4, bool TOUC
 int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N,
                 int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream, int splits = 1,
                 void* workspace = nullptr, int64_t blocks = 0, int first_block = 0) {
-  constexpr int kTileM = MODE == kQuads ? 256 : BM, kTileN = MODE == kQuads ? 256 : BN;
+  constexpr bool kParts = MODE == kQuads || MODE == kHalves;
+  constexpr int kTileM = kParts ? 256 : BM, kTileN = kParts ? 256 : BN;
   const int tiles_m = (int)ceil_div(M, kTileM), tiles_n = (int)ceil_div(N, kTileN);
   if ((int64_t)tiles_m * tiles_n > 0x7FFFFFFFll) return DT_ERR_INVALID_SHAPE;  // one workgroup per tile
   // NST K-steps: panels + scale slots (1 KiB per operand and 128-element chunk of the step)
@@ -593,7 +598,7 @@ int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const ui
   }
   uint8_t* const ws = static_cast<uint8_t*>(workspace);  // ticket counters, then the parked accumulators
   int64_t grid = (int64_t)tiles_m * tiles_n * splits;
-  if (blocks > 0) grid = MODE == kQuads ? 32 * ceil_div(blocks, (int64_t)8) : blocks;
+  if (blocks > 0) grid = kParts ? (MODE == kQuads ? 32 : 16) * ceil_div(blocks, (int64_t)8) : blocks;
   kernel<<<(unsigned)grid, WAVES_M * WAVES_N * kWave, lds_bytes, stream>>>(
       a, b, sfa, sfb, (int)M, (int)N, (int)K, lda, ldb, static_cast<uint16_t*>(out), ldo, tiles_m, tiles_n,
       (ldo % 8 == 0 && aligned(out, 16)) ? 1 : 0, splits, ws ? reinterpret_cast<v4f*>(ws + kSplitTicketBytes) : nullptr,
@@ -674,16 +679,21 @@ int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb
     // MI355X, e4m3, us: 4096 x 5120 x 4096, 256 + 64 tiles, 97 -> 77; 4352^2 x 4096, 256 + 33, 97 -> 78;
     // 4096 x 4352 x 8192, 256 + 16, 177 -> 134; 6144^3, 512 + 64, 216 -> 186; 8448 x 8192^2, 1024 + 32,
     // 473 -> 436), two rounds of quadrants take as long as the round of tiles (4096 x 6144 x 4096,
-    // 256 + 128: 97 -> 96).  The results are the same bits either way.
+    // 256 + 128: 97 -> 96).  Up to half a round of leftover tiles runs as 256 x 128 halves, a round of
+    // which takes 0.8 of a round of tiles (the same shape 97 -> 87.5; 8192 x 5120 x 8192, 512 + 128,
+    // 273 -> 258).  The results are the same bits either way.
     const int cus = device_facts().cu_count;
     const int64_t rounds = tiles256 / cus, left = tiles256 % cus;
     const int tail = tuning("gemm.tail_quads");
-    if (variant == 0 && tail != 0 && rounds >= 1 && left > 0 && cus % 8 == 0 && (tail == 2 || 4 * left <= cus)) {
+    if (variant == 0 && tail != 0 && rounds >= 1 && left > 0 && cus % 8 == 0 && (tail >= 2 || 2 * left <= cus)) {
       const int st = launch_gemm<256, 256, 2, 2, 2, FP4, true>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s, 1, nullptr,
                                                                 rounds * cus);
       if (st != DT_OK) return st;
-      return launch_gemm<128, 128, 2, 2, 4, FP4, false, kQuads>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s, 1, nullptr,
-                                                                left, (int)(rounds * cus));
+      if (tail == 2 || (tail == 1 && 4 * left <= cus))
+        return launch_gemm<128, 128, 2, 2, 4, FP4, false, kQuads>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s, 1, nullptr,
+                                                                  left, (int)(rounds * cus));
+      return launch_gemm<256, 128, 2, 2, 3, FP4, false, kHalves>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s, 1, nullptr,
+                                                                 left, (int)(rounds * cus));
     }
     return launch_gemm<256, 256, 2, 2, 2, FP4, true>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
   }

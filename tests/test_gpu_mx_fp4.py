@@ -89,17 +89,17 @@ def test_mx_fp4_gemm_split_k(d, cabi, splits, size):
 
 
 def test_mx_fp4_gemm_leftover_tiles_as_quadrants(d, cabi):
-    """272 tiles of 256 x 256: one round on the big kernel, 16 tiles as 128 x 128 quadrants; the same
+    """272 tiles of 256 x 256: one round on the big kernel, 16 tiles as 128 x 128 quadrants or as 256 x 128 halves; the same
     bits as the big kernel alone (with a half-filled last K-step: 384 = 1.5 steps)"""
     size = (4352, 384, 4096)
     outs = []
-    for tail in (2, 0):
+    for tail in (2, 0, 3):
         cabi.set_tuning("gemm.tail_quads", tail)
         try:
             outs.append(_check(d, *size, 1500, "randn"))
         finally:
             cabi.set_tuning("gemm.tail_quads", 1)
-    assert torch.equal(outs[0], outs[1])
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[2], outs[1])
 
 
 def test_mx_fp4_gemm_bit_exact_when_sums_fit_fp32(d):
