@@ -672,6 +672,12 @@ int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb
     if (variant == 8) return launch_gemm<256, 256, 2, 4, 2, false, true>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
   }
   if (big && variant == 7) return launch_gemm<256, 256, 2, 2, 2, FP4, false>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  // Between a quarter and half a round of 256 x 256 tiles: as 256 x 128 halves they fill the chip
+  // once (0.8 of a round of tiles), as 128 x 128 tiles they would take two rounds (2 x 0.55)
+  if (variant == 0 && tuning("gemm.tail_quads") != 0 && 4 * tiles256 > device_facts().cu_count &&
+      2 * tiles256 <= device_facts().cu_count)
+    return launch_gemm<256, 128, 2, 2, 3, FP4, false, kHalves>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s, 1, nullptr,
+                                                               tiles256, 0);
   if (big) {
     // Whole rounds of the chip on 256 x 256 tiles; what is left over would keep the chip for another
     // full round however few tiles it is.  When its quadrants fit the chip at once it runs as

@@ -210,7 +210,8 @@ def test_mx_gemm_split_k(d, cabi, splits, size):
         cabi.set_tuning("gemm.split_k", 0)
 
 
-@pytest.mark.parametrize("size", [(4352, 256, 4096), (4100, 256, 4360), (4352, 384, 4352), (8200, 128, 4104)],
+@pytest.mark.parametrize("size", [(4352, 256, 4096), (4100, 256, 4360), (4352, 384, 4352), (8200, 128, 4104),
+                                  (2304, 128, 2304), (2200, 256, 2312)],  # the last two: 81 and 90 tiles, halves only
                          ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
 def test_mx_gemm_leftover_tiles_as_quadrants(d, cabi, size):
     """more 256 x 256 tiles than CUs: whole rounds on the big kernel, the tiles left over as 128 x 128
