@@ -294,6 +294,16 @@ def extra_kernels(torch, cabi, util, dev, K, W, gemm_only=False):
     rows.append({"kernel": "mx_fp8_bf16", "workload": "config 5: 8192^3 e4m3 x e4m3, E8M0 block-32 scales -> bf16",
                  "bound": "mfma", "avg_us": round(us, 2), "achieved_TFLOPs": round(tf, 1),
                  "frac_of_fp8_peak": round(tf / FP8_PEAK_TFLOPS, 4), "flops": flops})
+    # two shapes off the 8192^3 grid, on row slices of the same operands (blocked scales are
+    # stored by 128-row chunks, so a row prefix of the operand owns a prefix of its scales)
+    for m_rows, n_rows, what in ((16, 8192, "16 rows: K shared between 4 workgroups per 128x128 tile"),
+                                 (1024, 8192, "128 tiles of 256x256 on 256 CUs: runs as 256 tiles of 256x128")):
+        sa_rows, sb_rows = -(-m_rows // 128) * 128 * (Kd // 32), -(-n_rows // 128) * 128 * (Kd // 32)
+        ops = (a_data[:m_rows], b_data[:n_rows], sfa[:sa_rows], sfb[:sb_rows], out[:m_rows, :n_rows])
+        us = time_launches(lambda i: cabi.mx_fp8_bf16(*ops), 1, max(20, K // 2), 10)
+        fl = 2.0 * m_rows * n_rows * Kd
+        rows.append({"kernel": "mx_fp8_bf16", "workload": f"{m_rows}x{n_rows}x{Kd} e4m3 ({what})", "bound": "mfma",
+                     "avg_us": round(us, 2), "achieved_TFLOPs": round(fl / (us * 1e-6) / 1e12, 1), "flops": fl})
     # MXFP4 GEMM, same shape: random e2m1 codes and scale bytes (no op of the path produces fp4)
     del a_data, b_data
     g = torch.Generator(device=dev).manual_seed(5)
