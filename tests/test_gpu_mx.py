@@ -227,6 +227,29 @@ def test_mx_gemm_leftover_tiles_as_quadrants(d, cabi, size):
     assert torch.equal(outs[1], outs[0]) and torch.equal(outs[2], outs[0])  # same K order per entry: the same bits
 
 
+@pytest.mark.parametrize("size", [(300, 1024, 264), (64, 8192, 512), (2304, 256, 2304), (4100, 256, 4360)],
+                         ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+def test_mx_gemm_strided_operands_and_output(d, cabi, size):
+    """operands that are column slices of wider matrices (row stride > K, data pointer off the
+    allocation's start) and an output that is a slice of a wider one: the same bits as with
+    contiguous tensors, on every launch plan"""
+    M, K, N = size
+    a_data, a_sc, b_data, b_sc = _operands(d, M, K, N, 1600 + M, "randn")
+    sa, sb = d.to_blocked(a_sc), d.to_blocked(b_sc)
+    want = d.mx_fp8_bf16(a_data, b_data.t(), sa, sb)
+    a_wide = torch.zeros((M, K + 384), dtype=torch.uint8, device="cuda").view(E4)
+    b_wide = torch.zeros((N, K + 640), dtype=torch.uint8, device="cuda").view(E4)
+    a_wide[:, 128:128 + K] = a_data
+    b_wide[:, 256:256 + K] = b_data
+    a_view, b_view = a_wide[:, 128:128 + K], b_wide[:, 256:256 + K]
+    assert a_view.stride(0) == K + 384 and not a_view.is_contiguous()
+    assert torch.equal(d.mx_fp8_bf16(a_view, b_view.t(), sa, sb), want)
+    out_wide = torch.full((M, N + 24), 7.0, dtype=torch.bfloat16, device="cuda")
+    cabi.mx_fp8_bf16(a_view, b_view, sa, sb, out_wide[:, 8:8 + N])
+    assert torch.equal(out_wide[:, 8:8 + N], want)
+    assert (out_wide[:, :8] == 7.0).all() and (out_wide[:, 8 + N:] == 7.0).all()  # nothing written outside
+
+
 def test_mx_gemm_split_k_workspace_rules(d, cabi):
     M, K, N = 32, 8192, 256  # 64 K-steps on 2 tiles: the library splits by itself
     a_data, a_sc, b_data, b_sc = _operands(d, M, K, N, 1200, "randn")
