@@ -275,6 +275,12 @@ def extra_kernels(torch, cabi, util, dev, K, W, gemm_only=False):
                 lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
                            torch.empty((256, 8192), dtype=torch.uint8, device=dev)),
                 lambda x, dd, s: cabi.mx_fp8_quantize(x, 0, False, e4, cabi.SCALE_PLAIN, dd, s))
+        # the cast that makes mx_fp4_bf16's operands: 2 B in, 1/2 B + 1/32 B out per element
+        hbm_row("mx_fp4_quantize rows, blocked scales", "bf16 [8192,8192] -> packed e2m1 + E8M0, scales in the GEMM's layout",
+                8192 * 8192 * (2 + 0.5 + 1 / 32),
+                lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 4096), dtype=torch.uint8, device=dev),
+                           torch.empty((nblk,), dtype=torch.uint8, device=dev)),
+                lambda x, dd, sc: cabi.mx_fp4_quantize(x, cabi.SCALE_BLOCKED, dd, sc))
 
     if not gemm_only:
         hbm_rows()

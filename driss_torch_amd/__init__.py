@@ -125,6 +125,14 @@ def mx_fp8_quantize_dual(input: Tensor, ScalarType: torch.dtype = torch.float8_e
     return ops.mx_fp8_quantize_dual(input, ScalarType, blocked)
 
 
+def mx_fp4_quantize(input: Tensor, blocked: bool = False) -> Tuple[Tensor, Tensor]:
+    """MXFP4 cast of ``input`` [M, N]: ``(packed e2m1 pairs [M, N/2] as uint8, E8M0 scales)``, blocks of
+    32 along the rows, the operands ``mx_fp4_bf16`` takes (the reference's test builds them with
+    torchao's ``MXTensor.to_mx(x, "fp4_e2m1", 32)``, test/test_mx.py:17-21).  ``blocked`` selects the
+    scale layout the GEMM reads; otherwise the flat scale tensor is the row-major [M, N/32] matrix."""
+    return ops.mx_fp4_quantize(input, blocked)
+
+
 def to_blocked(scale: Tensor) -> Tensor:
     """[R, C] E8M0 scale matrix -> flat blocked 128x4 layout (zero padded)."""
     return ops.to_blocked(scale)

@@ -83,6 +83,14 @@ def mx_fp8_quantize_dual_meta(x, fp8_type, blocked):
             torch.empty(shape_c, dtype=fp8_type, device=x.device), torch.empty((scale_c,), dtype=e8, device=x.device))
 
 
+@register_fake("DrissTorch::mx_fp4_quantize")
+def mx_fp4_quantize_meta(x, blocked):
+    m, n = x.shape
+    nscale = 128 * _ceil_div(m, 128) * 4 * _ceil_div(n // 32, 4) if blocked else m * (n // 32)
+    return (torch.empty((m, n // 2), dtype=torch.uint8, device=x.device),
+            torch.empty((nscale,), dtype=torch.float8_e8m0fnu, device=x.device))
+
+
 @register_fake("DrissTorch::to_blocked")
 def to_blocked_meta(scale):
     r, c = scale.shape

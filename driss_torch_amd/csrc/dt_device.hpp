@@ -165,6 +165,42 @@ template <int OUT>
 __device__ __forceinline__ uint32_t cvt_scaled_4x32(uint32_t a, uint32_t b, uint32_t c, uint32_t d, float scale) {
   return cvt_scaled_pair32<OUT, true>(cvt_scaled_pair32<OUT, false>(a, a, b, scale), c, d, scale);
 }
+// e2m1 (fp4): v_cvt_scalef32_pk_fp4_* converts two values of x / 2^(e-127) into one byte (first value
+// in the low nibble), round to nearest even, saturating at +-6; NaN becomes +-6, there being no NaN
+// code.  Measured on gfx950 against a host restatement: every bf16 pattern and 2^20 fp32 values,
+// scale bytes 0..254, bit-identical; the other three bytes of the word are left as they were.
+constexpr int DT_E2M1 = 2;  // internal output code (the public out-dtype enum covers the fp8 types)
+template <int IN>
+__device__ __forceinline__ uint32_t cvt_fp4_8x16(u32x4 w, float scale) {  // 8 elements -> 4 bytes
+  static_assert(IN == DT_BF16 || IN == DT_F16, "16-bit inputs");
+  // Each word goes through an empty asm first: handed the words of a 16-byte vector directly, hipcc
+  // (ROCm 7.2) selects the vector's FIRST word as the source of all four conversions.
+  uint32_t x = w.x, y = w.y, z = w.z, v = w.w;
+  asm("" : "+v"(x));
+  asm("" : "+v"(y));
+  asm("" : "+v"(z));
+  asm("" : "+v"(v));
+  uint32_t r = 0;
+  if constexpr (IN == DT_BF16) {
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(r, __builtin_bit_cast(v2bf16, x), scale, 0);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(r, __builtin_bit_cast(v2bf16, y), scale, 1);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(r, __builtin_bit_cast(v2bf16, z), scale, 2);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(r, __builtin_bit_cast(v2bf16, v), scale, 3);
+  } else {
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(r, __builtin_bit_cast(v2f16, x), scale, 0);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(r, __builtin_bit_cast(v2f16, y), scale, 1);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(r, __builtin_bit_cast(v2f16, z), scale, 2);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(r, __builtin_bit_cast(v2f16, v), scale, 3);
+  }
+  return r;
+}
+__device__ __forceinline__ uint32_t cvt_fp4_4x32(u32x4 w, float scale) {  // 4 elements -> 2 bytes (low half)
+  uint32_t r = 0;
+  r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, as_f32(w.x), as_f32(w.y), scale, 0);
+  r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, as_f32(w.z), as_f32(w.w), scale, 1);
+  return r;
+}
+
 // Product x*scale under the three rounding modes of dt_round_mode.  `sb` is the scale
 // already rounded for the mode (bf16-rounded for mode 2), so modes 1 and 2 share code.
 template <bool ROUND_PRODUCT_TO_BF16>

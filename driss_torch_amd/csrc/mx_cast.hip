@@ -191,6 +191,50 @@ extern "C" int dt_mx_fp8_quantize_dual(const void* x, int in_dtype, int64_t rows
   return dt_mx_fp8_quantize(x, in_dtype, rows, cols, 0, 1, out_dtype, scale_layout, data_cols_t, scale_cols_t, stream);
 }
 
+namespace {
+// MXFP4: the row-wise kernel with the e2m1 output code (same walk over the blocks, same scale stores)
+template <int IN, int LAYOUT>
+int launch_mx_fp4(const MxArgs& a) {
+  const int64_t nblocks = a.rows * a.cols / 32;
+  const int64_t nsuper = ceil_div(nblocks, (int64_t)64);
+  int64_t waves = (int64_t)device_facts().cu_count * tuning("mx.blocks_per_cu") * (kBlock / kWave);
+  if (waves > nsuper) waves = nsuper;
+  const unsigned grid = (unsigned)ceil_div(waves, (int64_t)(kBlock / kWave));
+  if constexpr (LAYOUT == DT_SCALE_BLOCKED) {
+    if (a.rows % 128 == 0 && a.cols % 512 == 0 && tuning("mx.row_band4")) {
+      mx_row_kernel<IN, DT_E2M1, LAYOUT, true><<<grid, kBlock, 0, a.stream>>>(a.x, (uint32_t)nblocks, (uint32_t)(a.cols / 32),
+                                                                             a.data, a.scale);
+      return launch_status();
+    }
+  }
+  mx_row_kernel<IN, DT_E2M1, LAYOUT><<<grid, kBlock, 0, a.stream>>>(a.x, (uint32_t)nblocks, (uint32_t)(a.cols / 32), a.data,
+                                                                   a.scale);
+  return launch_status();
+}
+}  // namespace
+
+extern "C" int dt_mx_fp4_quantize(const void* x, int in_dtype, int64_t rows, int64_t cols, int scale_layout, void* data,
+                                  uint8_t* scale, dt_stream_t stream) {
+  if (in_dtype != DT_F32 && in_dtype != DT_BF16 && in_dtype != DT_F16) return DT_ERR_INVALID_DTYPE;
+  if (scale_layout != DT_SCALE_PLAIN && scale_layout != DT_SCALE_BLOCKED) return DT_ERR_INVALID_MODE;
+  if (rows < 0 || cols < 0 || cols % 32 != 0) return DT_ERR_INVALID_SHAPE;
+  if (rows * cols / 32 >= (1ll << 28)) return DT_ERR_INVALID_SHAPE;  // block indices are 32 bits wide in the kernel
+  if (rows == 0 || cols == 0) return DT_OK;
+  if (!x || !data || !scale) return DT_ERR_NULL_POINTER;
+  if (!dt::aligned(x, 16) || !dt::aligned(data, 4)) return DT_ERR_MISALIGNED;
+  hipStream_t s = dt::as_hip(stream);
+  if (scale_layout == DT_SCALE_BLOCKED) {
+    if (int st = zero_blocked_padding(scale, rows, cols / 32, s)) return st;
+  }
+  MxArgs a{x, rows, cols, 1, 0, static_cast<uint8_t*>(data), scale, s};
+  const bool blocked = scale_layout == DT_SCALE_BLOCKED;
+  switch (in_dtype) {
+    case DT_F32: return blocked ? launch_mx_fp4<DT_F32, DT_SCALE_BLOCKED>(a) : launch_mx_fp4<DT_F32, DT_SCALE_PLAIN>(a);
+    case DT_BF16: return blocked ? launch_mx_fp4<DT_BF16, DT_SCALE_BLOCKED>(a) : launch_mx_fp4<DT_BF16, DT_SCALE_PLAIN>(a);
+    default: return blocked ? launch_mx_fp4<DT_F16, DT_SCALE_BLOCKED>(a) : launch_mx_fp4<DT_F16, DT_SCALE_PLAIN>(a);
+  }
+}
+
 extern "C" int dt_to_blocked(const uint8_t* scale, int64_t R, int64_t C, uint8_t* out, dt_stream_t stream) {
   if (R < 0 || C < 0) return DT_ERR_INVALID_SHAPE;
   if (R == 0 || C == 0) return DT_OK;

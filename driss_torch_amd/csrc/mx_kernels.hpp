@@ -46,6 +46,18 @@ struct MxScale {
 };
 template <int OUT>
 __device__ __forceinline__ MxScale<OUT> mx_scale_from_absbits(uint32_t absbits) {
+  if constexpr (OUT == DT_E2M1) {
+    // MXFP4: shared exponent floor(log2(max)) - 2 (2 = exponent of e2m1's largest value, 6), taken
+    // from the exponent field; an infinite maximum reads as field 255 (byte 253)
+    const int be = (int)(absbits >> 23);
+    const int b = be < 2 ? 0 : (be - 2 > 254 ? 254 : be - 2);
+    MxScale<OUT> r;
+    r.nan = absbits > 0x7F800000u;
+    r.byte = r.nan ? 255u : (uint32_t)b;
+    r.mult = as_f32((uint32_t)(254 - b) << 23);
+    r.scale = as_f32((uint32_t)b << 23);
+    return r;
+  }
   constexpr int kTargetPow2 = OUT == DT_E5M2 ? 15 : 8;
   const int be = (int)(absbits >> 23);
   const int mant_nz = (absbits & 0x7FFFFFu) ? 1 : 0;
@@ -181,7 +193,17 @@ __global__ __launch_bounds__(kBlock) void mx_row_kernel(const void* __restrict__
       const MxScale<OUT> s = mx_scale_from_absbits<OUT>(m);
       if ((lane % LPB) == c) mybyte = s.byte;
       if (vi < nvec) {
-        if constexpr (IN == DT_F32) {
+        if constexpr (OUT == DT_E2M1) {
+          // two elements per byte: a vector leaves as 4 bytes (16-bit inputs) or 2 (fp32); a block
+          // with a NaN gets 0x7 in every nibble under its NaN scale
+          if constexpr (IN == DT_F32) {
+            const uint32_t r = cvt_fp4_4x32(w[c], s.scale);
+            reinterpret_cast<uint16_t*>(data)[vi] = (uint16_t)(s.nan ? 0x7777u : r);
+          } else {
+            const uint32_t r = cvt_fp4_8x16<IN>(w[c], s.scale);
+            st_words(reinterpret_cast<uint32_t*>(data) + vi, s.nan ? 0x77777777u : r);
+          }
+        } else if constexpr (IN == DT_F32) {
           const uint32_t r = cvt_scaled_4x32<OUT>(w[c].x, w[c].y, w[c].z, w[c].w, s.scale);
           st_words(reinterpret_cast<uint32_t*>(data) + vi, s.nan ? 0x7F7F7F7Fu : r);
         } else {

@@ -184,7 +184,8 @@ def fp4_unpack(packed: torch.Tensor) -> torch.Tensor:
 
 
 def mx_fp4_quantize(x: torch.Tensor):
-    """Test-operand generator: fp32 [R, C] -> (packed e2m1 [R, C/2] uint8, E8M0 [R, C/32] uint8)."""
+    """MXFP4 cast of [R, C] (any float dtype; widened to fp32, which is exact) -> (packed e2m1 [R, C/2]
+    uint8, E8M0 [R, C/32] uint8)."""
     x = _cpu(x.float())
     R, Cc = x.shape
     data = torch.empty((R, Cc // 2), dtype=torch.uint8)

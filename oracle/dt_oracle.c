@@ -29,9 +29,14 @@
  * known-answer vectors in tests/golden/; amax/scale/cast against the eager formulation;
  * the MX exponent against ceil(log2) in exact (float64 / integer) arithmetic; to_blocked
  * against the view/permute formulation; the GEMM against brute force and float64 matmul.
- * The e2m1 decode is pinned by the eight magnitudes of the OCP table and the sign bit; the fp4
- * quantizer below only manufactures test operands (floor-exponent scaling as in the OCP
- * specification) and is "parity unpinned" against torchao's to_mx, which no op of the path calls.
+ * The e2m1 decode is pinned by the eight magnitudes of the OCP table and the sign bit, the e2m1
+ * encode by brute force over a dense sweep (nearest grid value, ties to the even code, saturation at
+ * 6), the fp4 quantizer's exponent by floor(log2) in exact arithmetic and by the invariant that the
+ * scaled block maximum lies in [4, 8) (so it rounds to 4 or 6 and nothing but rounding saturates).
+ * Against torchao's to_mx (what the reference's GEMM test calls for its operands, test/test_mx.py:20-21)
+ * the quantizer is "parity unpinned": its floor-mode formula is restated from the OCP specification
+ * and the public torchao source as recalled; its NaN / infinity / zero-block bytes are this build's
+ * documented choices.
  * Documented choices where the third-party oracle (torchao) is version dependent and no
  * vector in the reference pins it ("parity unpinned" corners): a block holding a NaN gets
  * scale byte 255 and an all-NaN payload; scale byte 0 decodes to 2^-127 (its E8M0 value);
@@ -439,22 +444,31 @@ DTO_EXPORT void dto_fp4_unpack(const uint8_t* packed, int64_t R, int64_t C, floa
     }
 }
 
-/* Test-operand generator: fp32 [R, C] -> packed e2m1 [R, C/2] + E8M0 [R, C/32], shared
- * exponent floor(log2(blockmax)) - 2 (2 = emax of e2m1), zero blocks get byte 0. */
+/* MXFP4 cast: fp32 [R, C] -> packed e2m1 [R, C/2] + E8M0 [R, C/32].  torchao's to_mx(x, "fp4_e2m1",
+ * 32) in its default (floor) scale mode as called at test/test_mx.py:20-21: shared exponent =
+ * exponent field of max|x| - 127 - 2 (2 = exponent of 6, e2m1's largest value), clamped to
+ * [-127, 127]; payload = e2m1 RNE, saturating, of x * 2^-exponent.  A zero or subnormal maximum gives
+ * byte 0, an infinite one field 255 -> byte 253; a block that holds a NaN gives byte 255 and the
+ * payload 0x7 in every nibble (e2m1 has no NaN; the scale carries it). */
 DTO_EXPORT void dto_mx_fp4_quantize(const float* x, int64_t R, int64_t C, uint8_t* data, uint8_t* scale) {
   for (int64_t r = 0; r < R; ++r)
     for (int64_t kb = 0; kb < C / 32; ++kb) {
       const float* p = x + r * C + kb * 32;
-      float m = 0.f;
-      for (int i = 0; i < 32; ++i) m = fmaxf(m, fabsf(p[i]));
-      int e = -127;
-      if (m > 0.f) { int ex; frexpf(m, &ex); e = ex - 1 - 2; }
-      if (e < -127) e = -127;
-      if (e > 127) e = 127;
-      scale[r * (C / 32) + kb] = (uint8_t)(e + 127);
+      uint32_t m = 0;
+      int has_nan = 0;
+      for (int i = 0; i < 32; ++i) {
+        uint32_t a = f2u(p[i]) & 0x7FFFFFFFu;
+        if (a > 0x7F800000u) has_nan = 1;
+        if (a > m) m = a;
+      }
+      int b = (int)(m >> 23) - 2;
+      if (b < 0) b = 0;
+      if (b > 254) b = 254;
+      const int e = b - 127;
+      scale[r * (C / 32) + kb] = has_nan ? 255 : (uint8_t)b;
       for (int i = 0; i < 32; i += 2) {
         uint8_t lo = dto_f32_to_e2m1(ldexpf(p[i], -e)), hi = dto_f32_to_e2m1(ldexpf(p[i + 1], -e));
-        data[r * (C / 2) + kb * 16 + i / 2] = (uint8_t)(lo | (hi << 4));
+        data[r * (C / 2) + kb * 16 + i / 2] = has_nan ? 0x77 : (uint8_t)(lo | (hi << 4));
       }
     }
 }

@@ -166,6 +166,32 @@ def fp4_unpack(packed_u8: torch.Tensor) -> torch.Tensor:
     return torch.stack([lo, hi], dim=-1).reshape(packed_u8.shape[0], -1)
 
 
+def mx_fp4_quantize(x: torch.Tensor, block: int = 32):
+    """MXFP4 cast in eager form: torchao's ``to_mx(x, "fp4_e2m1", 32)`` in its default (floor) scale mode,
+    as called at test/test_mx.py:20-21, restated with torch ops (torchao is not importable here).
+    -> (packed e2m1 [R, C/2] uint8, E8M0 [R, C/32] uint8).  Special blocks as in oracle/dt_oracle.c."""
+    R, Cc = x.shape
+    v = x.to(torch.float32).reshape(R, Cc // block, block)
+    has_nan = torch.isnan(v).any(-1)
+    amax = torch.where(torch.isnan(v), torch.zeros_like(v), v.abs()).amax(-1)
+    field = (amax.view(torch.int32) >> 23) & 0xFF            # floor(log2) + 127 for normal numbers
+    byte = torch.clamp(field - 2, 0, 254)
+    scaled = v.double() * torch.exp2((127 - byte).double()).unsqueeze(-1)   # exact in float64
+    grid = torch.tensor(E2M1_VALUES, dtype=torch.float64)
+    mids = (grid[:-1] + grid[1:]) / 2
+    a = scaled.abs()
+    code = torch.bucketize(a, mids, right=False)             # a == mid goes to the lower code ...
+    tie_up = torch.zeros_like(code, dtype=torch.bool)
+    for i, m in enumerate(mids.tolist()):                    # ... unless the lower code is odd
+        tie_up |= (a == m) & (i % 2 == 1)
+    code = torch.where(tie_up, code + 1, code)
+    code = torch.where(torch.isnan(a), torch.full_like(code, 7), code)
+    code = (code | torch.where(torch.signbit(scaled), 8, 0)).to(torch.uint8)
+    code = torch.where(has_nan.unsqueeze(-1), torch.full_like(code, 7), code).reshape(R, Cc)
+    packed = code[:, 0::2] | (code[:, 1::2] << 4)
+    return packed, torch.where(has_nan, torch.full_like(byte, 255), byte).to(torch.uint8)
+
+
 def mx_fp4_dequant(packed_u8: torch.Tensor, scale_u8: torch.Tensor, block: int = 32) -> torch.Tensor:
     v = fp4_unpack(packed_u8)
     R, Cc = v.shape

@@ -159,6 +159,16 @@ def test_mx_casts_past_2_32_elements(d):
             assert torch.equal(o[3].view(torch.uint8), scale_t.view(torch.uint8))
         del o
 
+    # the MXFP4 cast of the same tensor (packed pairs: column period base_c / 2)
+    fd, fs = co.mx_fp4_quantize(base)
+    d4, s4 = d.mx_fp4_quantize(x)
+    assert _tiles_equal(d4, fd, rep_r, rep_c)
+    assert _tiles_equal(s4.view(torch.uint8).view(R, C // 32), fs, rep_r, rep_c)
+    d4b, s4b = d.mx_fp4_quantize(x, True)
+    assert torch.equal(d4b, d4)
+    assert torch.equal(s4b.view(torch.uint8).cpu(), co.to_blocked(s4.view(torch.uint8).view(R, C // 32).cpu()))
+    del d4, s4, d4b, s4b
+
     # a block past element 2^32 that differs from its period, in both directions
     r0, c0 = R - 32, C - 32
     x[r0 + 5, c0 + 7] = 1.0e4

@@ -1,6 +1,7 @@
 """GPU parity of mx_fp4_bf16 (e2m1 operands, E8M0 block-32 scales) against the CPU oracle, on the
-reference's size list (test/test_mx.py:42-59 with format "fp4").  Operands come from the oracle's
-fp4 generator: the reference takes them from torchao's MXTensor, and no op of the path makes them."""
+reference's size list (test/test_mx.py:42-59 with format "fp4"), with operands from the oracle's MXFP4
+cast, and of mx_fp4_quantize (the device cast that makes such operands; the reference takes them from
+torchao's MXTensor) bit for bit against the same oracle."""
 import pytest
 import torch
 
@@ -190,3 +191,101 @@ def test_mx_fp4_gemm_full_size(d):
     ref, bound = da @ db.T, da.abs() @ db.abs().T
     got = out[rows.cuda()][:, cols.cuda()].cpu().double()
     assert ((got - ref).abs() <= bound * 2**-8).all()
+
+
+# --------------------------------------------------------------------------- MXFP4 cast
+def _check_fp4_cast(d, x):
+    data, scale = d.mx_fp4_quantize(x.cuda())
+    rd, rs = co.mx_fp4_quantize(x)
+    M, N = x.shape
+    assert data.dtype == torch.uint8 and data.shape == (M, N // 2) and scale.dtype == torch.float8_e8m0fnu
+    assert torch.equal(util.codes(scale).view(M, N // 32), rs)
+    assert torch.equal(data.cpu(), rd)
+    bdata, bscale = d.mx_fp4_quantize(x.cuda(), True)
+    assert torch.equal(bdata.cpu(), rd)
+    assert torch.equal(util.codes(bscale), co.to_blocked(rs))
+    return data, scale
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("shape", [(128, 32), (1, 64), (77, 96), (256, 512), (384, 1024), (130, 544), (2048, 4096)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+def test_mx_fp4_cast_against_oracle(d, in_dtype, shape):
+    g = util.gen(shape[0] + shape[1])
+    x = torch.randn(shape, generator=g) * torch.exp(2.0 * torch.randn(shape, generator=g))
+    if in_dtype == torch.float16:
+        x = x.clamp(-6.0e4, 6.0e4)
+    _check_fp4_cast(d, x.to(in_dtype))
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
+def test_mx_fp4_cast_special_blocks(d, in_dtype):
+    x = util.normal((128, 512), 41, in_dtype)
+    tiny = torch.finfo(in_dtype).tiny
+    x[0, :32] = 0.0
+    x[1, 32:64] = tiny / 4               # subnormal maximum
+    x[2, 5] = float("inf")
+    x[3, 40] = float("-inf")
+    x[4, 70] = float("nan")
+    x[5, 100] = float("nan")
+    x[5, 101] = float("inf")
+    x[6, :32] = torch.finfo(in_dtype).max
+    x[7, :32] = tiny
+    x[8, :32] = (torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0] * 4)).to(in_dtype)   # the grid's ties
+    x[9, :32] = -x[8, :32]
+    _check_fp4_cast(d, x)
+
+
+def test_mx_fp4_cast_every_bf16_pattern(d):
+    """all 65536 bf16 patterns as block members, under block maxima that put them below, inside and
+    above the e2m1 range (NaN patterns only in the NaN rows)"""
+    pats = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    finite = pats.clone()
+    finite[torch.isnan(pats) | torch.isinf(pats)] = 1.0
+    rows = []
+    for top in (2.0 ** -120, 2.0 ** -20, 0.5, 1.0, 6.0, 448.0, 2.0 ** 60, 3.0e38):
+        body = finite.float().view(2048, 32).clone()
+        body[:, 0] = top                      # the block maximum, unless a pattern is larger
+        rows.append(body.view(64, 1024))
+    rows.append(pats.float().view(64, 1024))  # with NaN and infinity patterns in place
+    x = torch.cat(rows).to(torch.bfloat16)
+    _check_fp4_cast(d, x)
+
+
+def test_mx_fp4_cast_feeds_the_gemm(d):
+    """cast -> blocked scales -> mx_fp4_bf16 against the float64 product of the dequantized operands
+    and, loosely, against the product of the inputs (e2m1 keeps 1-2 significant bits)"""
+    M, K, N = 256, 1024, 384
+    a, b = util.normal((M, K), 42), util.normal((N, K), 43)
+    ad, sa = d.mx_fp4_quantize(a.cuda(), True)
+    bd, sb = d.mx_fp4_quantize(b.cuda(), True)
+    out = d.mx_fp4_bf16(ad, bd.t(), sa, sb)
+    _, sa_plain = d.mx_fp4_quantize(a.cuda())
+    _, sb_plain = d.mx_fp4_quantize(b.cuda())
+    da = eager.mx_fp4_dequant(ad.cpu(), util.codes(sa_plain).view(M, K // 32))
+    db = eager.mx_fp4_dequant(bd.cpu(), util.codes(sb_plain).view(N, K // 32))
+    ref = da @ db.T
+    bound = da.abs() @ db.abs().T
+    assert ((out.cpu().double() - ref).abs() <= bound * 2**-8).all()
+    assert eager.compute_error(a.double() @ b.double().T, out.cpu().double()).item() > 15  # fp4 operands: ~18 dB
+
+
+def test_mx_fp4_cast_errors_and_compile(d, cabi):
+    x = util.normal((64, 128), 44).cuda()
+    with pytest.raises(RuntimeError):
+        d.mx_fp4_quantize(x[:, :48])                  # not contiguous
+    with pytest.raises(RuntimeError):
+        d.mx_fp4_quantize(x[:, :48].contiguous())     # 48 % 32
+    with pytest.raises(RuntimeError):
+        d.mx_fp4_quantize(x.double())
+    e_data, e_scale = d.mx_fp4_quantize(x[:0])
+    assert e_data.shape == (0, 64) and e_scale.numel() == 0
+    L = cabi.lib()
+    data = torch.empty(64 * 64 + 8, dtype=torch.uint8, device="cuda")
+    scale = torch.empty(64 * 4, dtype=torch.uint8, device="cuda")
+    assert L.dt_mx_fp4_quantize(x.data_ptr(), cabi.BF16, 64, 128, 0, data.data_ptr() + 2, scale.data_ptr(), None) == 4
+    assert L.dt_mx_fp4_quantize(x.data_ptr(), cabi.BF16, 64, 128, 2, data.data_ptr(), scale.data_ptr(), None) == 6
+    assert L.dt_mx_fp4_quantize(x.data_ptr(), 7, 64, 128, 0, data.data_ptr(), scale.data_ptr(), None) == 1
+    fn = torch.compile(lambda t: d.mx_fp4_quantize(t, True), fullgraph=True, backend="aot_eager")
+    got, want = fn(x), d.mx_fp4_quantize(x, True)
+    assert torch.equal(got[0], want[0]) and torch.equal(util.codes(got[1]), util.codes(want[1]))

@@ -65,6 +65,11 @@ def test_mx_casts_random_shapes(d, shape, in_dtype):
     x = _data(shape, shape[0] * 17 + shape[1], in_dtype)
     g = x.cuda()
     rows, cols = shape
+    if cols % 32 == 0:  # the MXFP4 cast, plain and blocked scales
+        fd, fs = co.mx_fp4_quantize(x)
+        for blocked in (False, True):
+            data, scale = d.mx_fp4_quantize(g, blocked)
+            assert torch.equal(data.cpu(), fd) and torch.equal(util.codes(scale), (co.to_blocked(fs) if blocked else fs).flatten())
     for fp8 in (E4, E5):
         if cols % 32 == 0:
             rd, rs = co.mx_quantize(x, axis=1, transpose=False, out_dtype=fp8)

@@ -211,6 +211,40 @@ def test_fp4_operand_generator_properties():
     assert torch.equal(eager.mx_fp4_dequant(d2, s2).float(), deq)
 
 
+def test_fp4_quantize_c_vs_eager_and_special_blocks():
+    """the C restatement against the torch one on wide-range data in fp32 and bf16, and the documented
+    special blocks: zero and subnormal maxima (byte 0), infinity (byte 253, payload saturates), NaN
+    (byte 255, every nibble 7), the largest and smallest normal maxima, exact ties"""
+    g = util.gen(36)
+    x = torch.randn(96, 256, generator=g) * torch.exp(3.0 * torch.randn(96, 256, generator=g))
+    x[0, :32] = 0.0
+    x[1, :32] = 1e-41                      # subnormal block
+    x[2, 5] = float("inf")
+    x[3, 40] = float("-inf")
+    x[4, 70] = float("nan")
+    x[5, :32] = torch.finfo(torch.float32).max
+    x[6, :32] = torch.finfo(torch.float32).tiny * 3
+    x[7, :32] = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0] * 4) * 1.0   # ties of the grid at scale 1 (max 6 -> byte 127)
+    x[7, 31] = -5.0
+    for t in (x, x.to(torch.bfloat16)):
+        dc, sc = co.mx_fp4_quantize(t)
+        de, se = eager.mx_fp4_quantize(t)
+        assert torch.equal(sc, se) and torch.equal(dc, de)
+    d, s = co.mx_fp4_quantize(x)
+    assert s[0, 0] == 0 and (d[0, :16] == 0).all()
+    assert s[1, 0] == 0 and (d[1, :16] == 0).all()
+    assert s[2, 0] == 253 and (d[2, 2] & 15) == 0 and (d[2, 2] >> 4) == 7      # element 5 = +inf -> 6
+    assert s[3, 1] == 253 and (d[3, 20] & 15) == 15                            # element 40 = -inf -> -6
+    assert s[4, 2] == 255 and (d[4, 32:48] == 0x77).all()
+    assert s[5, 0] == 252 and (d[5, :16] == 0x77).all()                        # max = 1.99.. * 2^127 -> 7.99.. -> saturates at 6
+    assert s[6, 0] == 0
+    assert s[7, 0] == 127
+    # 0.25 -> 0 (tie to even code 0), 0.75 -> 1.0 (code 2), 1.25 -> 1.0, 1.75 -> 2.0 (code 4), 2.5 -> 2.0, 3.5 -> 4.0 (code 6), 5 -> 4.0, 6 -> 6
+    assert [int(d[7, 0]) & 15, int(d[7, 0]) >> 4, int(d[7, 1]) & 15, int(d[7, 1]) >> 4] == [0, 2, 2, 4]
+    assert [int(d[7, 2]) & 15, int(d[7, 2]) >> 4, int(d[7, 3]) & 15, int(d[7, 3]) >> 4] == [4, 6, 6, 7]
+    assert int(d[7, 15]) >> 4 == 8 | 6                                          # -5 -> -4
+
+
 def test_fp4_gemm_ref_against_float64_matmul_and_brute_force():
     M, N, K = 70, 52, 384
     a, sa = co.mx_fp4_quantize(util.normal((M, K), 34, torch.float32))
