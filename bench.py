@@ -310,13 +310,10 @@ def extra_kernels(torch, cabi, util, dev, K, W, gemm_only=False):
         fl = 2.0 * m_rows * n_rows * Kd
         rows.append({"kernel": "mx_fp8_bf16", "workload": f"{m_rows}x{n_rows}x{Kd} e4m3 ({what})", "bound": "mfma",
                      "avg_us": round(us, 2), "achieved_TFLOPs": round(fl / (us * 1e-6) / 1e12, 1), "flops": fl})
-    # MXFP4 GEMM, same shape: random e2m1 codes and scale bytes (no op of the path produces fp4)
+    # MXFP4 GEMM, same shape: the MXFP4 cast of the same N(0,1) operands, scales blocked by the cast
     del a_data, b_data
-    g = torch.Generator(device=dev).manual_seed(5)
-    a4 = torch.randint(0, 256, (M, Kd // 2), generator=g, dtype=torch.uint8, device=dev)
-    b4 = torch.randint(0, 256, (N, Kd // 2), generator=g, dtype=torch.uint8, device=dev)
-    s4a = torch.randint(120, 134, (sfa.numel(),), generator=g, dtype=torch.uint8, device=dev)
-    s4b = torch.randint(120, 134, (sfb.numel(),), generator=g, dtype=torch.uint8, device=dev)
+    a4, s4a = cabi.mx_fp4_quantize(rnd((M, Kd), bf16, 1), cabi.SCALE_BLOCKED)
+    b4, s4b = cabi.mx_fp4_quantize(rnd((N, Kd), bf16, 2), cabi.SCALE_BLOCKED)
     us = time_launches(lambda i: cabi.mx_fp4_bf16(a4, b4, s4a, s4b, out), 1, max(20, K // 2), max(30, W))
     tf = flops / (us * 1e-6) / 1e12
     rows.append({"kernel": "mx_fp4_bf16", "workload": "8192^3 e2m1 x e2m1, E8M0 block-32 scales -> bf16",
