@@ -44,6 +44,7 @@ SIGNATURES = {
     "dt_mx_fp8_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     "dt_mx_fp4_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     "dt_mx_gemm_workspace_bytes": (_sz, []),
+    "dt_mx_gemm_workspace_init": (_i32, [_vp, _sz, _vp]),
     "dt_mx_fp8_bf16_ws": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "dt_mx_fp4_bf16_ws": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "dt_set_tuning": (_i32, [_cp, _i32]),
@@ -114,7 +115,8 @@ def gemm_workspace(device=None) -> torch.Tensor:
     key = (dev.index, _stream())
     ws = _gemm_workspaces.get(key)
     if ws is None:
-        ws = torch.zeros(lib().dt_mx_gemm_workspace_bytes(), dtype=torch.uint8, device=dev)
+        ws = torch.empty(lib().dt_mx_gemm_workspace_bytes(), dtype=torch.uint8, device=dev)
+        _check(lib().dt_mx_gemm_workspace_init(ws.data_ptr(), ws.numel(), _stream()), "dt_mx_gemm_workspace_init")
         _gemm_workspaces[key] = ws
     return ws
 

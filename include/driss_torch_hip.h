@@ -208,9 +208,11 @@ DT_API int dt_mx_fp4_quantize(const void* x, int in_dtype, int64_t rows, int64_t
  * dt_mx_gemm_workspace_bytes() bytes, 256-byte aligned.  With it a problem whose output tiles
  * leave most CUs idle (few rows or columns, long K) shares K between several workgroups per
  * tile; the result does not depend on their timing.  The first 1 KiB of the workspace must be
- * zero before the first call and is left zero by every call; calls that may overlap on the
- * device need workspaces of their own.  workspace == NULL behaves as the plain entry point. */
+ * zero before the first call (dt_mx_gemm_workspace_init, or any memset) and is left zero by
+ * every call; calls that may overlap on the device need workspaces of their own.
+ * workspace == NULL behaves as the plain entry point.                                     */
 DT_API size_t dt_mx_gemm_workspace_bytes(void);
+DT_API int dt_mx_gemm_workspace_init(void* workspace, size_t workspace_bytes, dt_stream_t stream);
 DT_API int dt_mx_fp8_bf16_ws(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb,
                              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, void* out,
                              int64_t ldo, void* workspace, size_t workspace_bytes, dt_stream_t stream);

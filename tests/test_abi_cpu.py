@@ -73,6 +73,9 @@ def test_host_validation_without_gpu():
     assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 128, 512, 8192, 8192, 1 << 25, fake, 512, None) == 2
     # the entry points with a split-K workspace: same checks, plus the workspace's alignment
     assert L.dt_mx_gemm_workspace_bytes() >= 1024 + 128 * 128 * 4
+    assert L.dt_mx_gemm_workspace_init(None, 1 << 20, None) == 3
+    assert L.dt_mx_gemm_workspace_init(fake, 512, None) == 5
+    assert L.dt_mx_gemm_workspace_init(fake + 16, 1 << 20, None) == 4
     assert L.dt_mx_fp8_bf16_ws(fake, fake, fake, fake, 128, 128, 96, 96, 96, fake, 128, fake, 1 << 20, None) == 2
     assert L.dt_mx_fp8_bf16_ws(fake, fake, fake, fake, 128, 128, 128, 128, 128, fake, 128, fake + 16, 1 << 20, None) == 4
     assert L.dt_mx_fp4_bf16_ws(fake, fake, fake, fake, 128, 128, 256, 128, 128, fake, 128, fake + 16, 1 << 20, None) == 4

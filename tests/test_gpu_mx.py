@@ -261,7 +261,8 @@ def test_mx_gemm_split_k_workspace_rules(d, cabi):
         assert eager.compute_error(ref, got.cpu().double()).item() > 50
     L = cabi.lib()
     out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
-    ws = torch.zeros(L.dt_mx_gemm_workspace_bytes() + 256, dtype=torch.uint8, device="cuda")
+    ws = torch.full((L.dt_mx_gemm_workspace_bytes() + 256,), 0xAB, dtype=torch.uint8, device="cuda")
+    assert L.dt_mx_gemm_workspace_init(ws.data_ptr(), ws.numel(), None) == 0  # zeroes the ticket counters
     args = (a_data.data_ptr(), b_data.data_ptr(), sa.data_ptr(), sb.data_ptr(), M, N, K, K, K, out.data_ptr(), N)
     assert L.dt_mx_fp8_bf16_ws(*args, ws.data_ptr() + 8, ws.numel() - 8, None) == 4  # misaligned workspace
     # a workspace too small for any split: the product is computed without one
