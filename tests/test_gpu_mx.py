@@ -250,6 +250,26 @@ def test_mx_gemm_strided_operands_and_output(d, cabi, size):
     assert (out_wide[:, :8] == 7.0).all() and (out_wide[:, 8 + N:] == 7.0).all()  # nothing written outside
 
 
+def test_mx_gemm_split_k_on_two_streams(d):
+    """split-K products issued alternately on two streams (each stream has its own ticket counters and
+    parking space in the torch shim): every result equals the one computed alone"""
+    M, K, N = 48, 8192, 384
+    ops = []
+    for seed in (1700, 1710):
+        a_data, a_sc, b_data, b_sc = _operands(d, M, K, N, seed, "randn")
+        ops.append((a_data, b_data.t(), d.to_blocked(a_sc), d.to_blocked(b_sc)))
+    want = [d.mx_fp8_bf16(*o) for o in ops]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = []
+    for rep in range(12):
+        with torch.cuda.stream(streams[rep % 2]):
+            got.append((rep % 2, d.mx_fp8_bf16(*ops[rep % 2])))
+    torch.cuda.synchronize()
+    for which, out in got:
+        assert torch.equal(out, want[which])
+
+
 def test_mx_gemm_split_k_workspace_rules(d, cabi):
     M, K, N = 32, 8192, 256  # 64 K-steps on 2 tiles: the library splits by itself
     a_data, a_sc, b_data, b_sc = _operands(d, M, K, N, 1200, "randn")
