@@ -125,12 +125,14 @@ def mx_fp8_quantize_dual(input: Tensor, ScalarType: torch.dtype = torch.float8_e
     return ops.mx_fp8_quantize_dual(input, ScalarType, blocked)
 
 
-def mx_fp4_quantize(input: Tensor, blocked: bool = False) -> Tuple[Tensor, Tensor]:
-    """MXFP4 cast of ``input`` [M, N]: ``(packed e2m1 pairs [M, N/2] as uint8, E8M0 scales)``, blocks of
-    32 along the rows, the operands ``mx_fp4_bf16`` takes (the reference's test builds them with
-    torchao's ``MXTensor.to_mx(x, "fp4_e2m1", 32)``, test/test_mx.py:17-21).  ``blocked`` selects the
-    scale layout the GEMM reads; otherwise the flat scale tensor is the row-major [M, N/32] matrix."""
-    return ops.mx_fp4_quantize(input, blocked)
+def mx_fp4_quantize(input: Tensor, blocked: bool = False, axis: int = 1) -> Tuple[Tensor, Tensor]:
+    """MXFP4 cast of ``input`` [M, N]: ``(packed e2m1 pairs as uint8, E8M0 scales)``, the operands
+    ``mx_fp4_bf16`` takes (the reference's test builds them with torchao's
+    ``MXTensor.to_mx(x, "fp4_e2m1", 32)``, test/test_mx.py:17-21).  axis 1: blocks of 32 along the rows,
+    payload [M, N/2], scale matrix [M, N/32]; axis 0: blocks down the columns with the payload
+    transposed, [N, M/2] and [N, M/32], which equals the axis-1 cast of ``input.t().contiguous()``.
+    ``blocked`` selects the scale layout the GEMM reads; otherwise the flat scale tensor is row-major."""
+    return ops.mx_fp4_quantize(input, blocked, axis)
 
 
 def to_blocked(scale: Tensor) -> Tensor:

@@ -84,10 +84,11 @@ def mx_fp8_quantize_dual_meta(x, fp8_type, blocked):
 
 
 @register_fake("DrissTorch::mx_fp4_quantize")
-def mx_fp4_quantize_meta(x, blocked):
+def mx_fp4_quantize_meta(x, blocked, axis):
     m, n = x.shape
-    nscale = 128 * _ceil_div(m, 128) * 4 * _ceil_div(n // 32, 4) if blocked else m * (n // 32)
-    return (torch.empty((m, n // 2), dtype=torch.uint8, device=x.device),
+    outer, inner = (m, n) if axis % 2 == 1 else (n, m)
+    nscale = 128 * _ceil_div(outer, 128) * 4 * _ceil_div(inner // 32, 4) if blocked else outer * (inner // 32)
+    return (torch.empty((outer, inner // 2), dtype=torch.uint8, device=x.device),
             torch.empty((nscale,), dtype=torch.float8_e8m0fnu, device=x.device))
 
 

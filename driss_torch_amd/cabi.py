@@ -38,7 +38,7 @@ SIGNATURES = {
     "dt_dynamic_scaled_quant_rowwise": (_i32, [_vp, _i32, _i64, _i64, _i32, _vp, _vp, _vp, _vp]),
     "dt_mx_fp8_quantize": (_i32, [_vp, _i32, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
     "dt_mx_fp8_quantize_dual": (_i32, [_vp, _i32, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
-    "dt_mx_fp4_quantize": (_i32, [_vp, _i32, _i64, _i64, _i32, _vp, _vp, _vp]),
+    "dt_mx_fp4_quantize": (_i32, [_vp, _i32, _i64, _i64, _i32, _i32, _vp, _vp, _vp]),
     "dt_blocked_scale_bytes": (_i64, [_i64, _i64]),
     "dt_to_blocked": (_i32, [_vp, _i64, _i64, _vp, _vp]),
     "dt_mx_fp8_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
@@ -237,15 +237,17 @@ def mx_fp8_quantize_dual(x: torch.Tensor, out_dtype: torch.dtype = torch.float8_
     return dr, sr, dc, sc
 
 
-def mx_fp4_quantize(x: torch.Tensor, layout: int = 0, data=None, scale=None):
-    """x [R, C] -> (packed e2m1 [R, C/2] uint8, E8M0 bytes: [R, C/32] plain or flat blocked)"""
+def mx_fp4_quantize(x: torch.Tensor, layout: int = 0, data=None, scale=None, axis: int = 1):
+    """x [R, C] -> (packed e2m1 uint8, E8M0 bytes plain or flat blocked): axis 1 -> [R, C/2] and [R, C/32],
+    axis 0 -> the cast of x^T, [C, R/2] and [C, R/32]"""
     R, Cc = x.shape
-    data = torch.empty((R, Cc // 2), dtype=torch.uint8, device=x.device) if data is None else data
+    outer, inner = (R, Cc) if axis == 1 else (Cc, R)
+    data = torch.empty((outer, inner // 2), dtype=torch.uint8, device=x.device) if data is None else data
     if scale is None:
-        n = lib().dt_blocked_scale_bytes(R, Cc // 32) if layout == SCALE_BLOCKED else R * (Cc // 32)
+        n = lib().dt_blocked_scale_bytes(outer, inner // 32) if layout == SCALE_BLOCKED else outer * (inner // 32)
         scale = torch.empty((n,), dtype=torch.uint8, device=x.device)
-    _check(lib().dt_mx_fp4_quantize(x.data_ptr(), IN_DTYPE[x.dtype], R, Cc, layout, data.data_ptr(), scale.data_ptr(), _stream()),
-           "dt_mx_fp4_quantize")
+    _check(lib().dt_mx_fp4_quantize(x.data_ptr(), IN_DTYPE[x.dtype], R, Cc, axis, layout, data.data_ptr(), scale.data_ptr(),
+                                    _stream()), "dt_mx_fp4_quantize")
     return data, scale
 
 

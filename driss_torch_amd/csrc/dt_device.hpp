@@ -194,6 +194,32 @@ __device__ __forceinline__ uint32_t cvt_fp4_8x16(u32x4 w, float scale) {  // 8 e
   }
   return r;
 }
+// one pair into byte `sel` (0..3) of `old`
+template <int IN>
+__device__ __forceinline__ uint32_t cvt_fp4_pair16(uint32_t old, uint32_t pair, float scale, int sel) {
+  static_assert(IN == DT_BF16 || IN == DT_F16, "16-bit inputs");
+  asm("" : "+v"(pair));  // see cvt_fp4_8x16
+  if constexpr (IN == DT_BF16) {
+    const v2bf16 x = __builtin_bit_cast(v2bf16, pair);
+    return sel == 0 ? __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(old, x, scale, 0)
+         : sel == 1 ? __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(old, x, scale, 1)
+         : sel == 2 ? __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(old, x, scale, 2)
+                    : __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(old, x, scale, 3);
+  } else {
+    const v2f16 x = __builtin_bit_cast(v2f16, pair);
+    return sel == 0 ? __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(old, x, scale, 0)
+         : sel == 1 ? __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(old, x, scale, 1)
+         : sel == 2 ? __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(old, x, scale, 2)
+                    : __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(old, x, scale, 3);
+  }
+}
+__device__ __forceinline__ uint32_t cvt_fp4_pair32(uint32_t old, uint32_t a, uint32_t b, float scale, int sel) {
+  const float x = as_f32(a), y = as_f32(b);
+  return sel == 0 ? __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, x, y, scale, 0)
+       : sel == 1 ? __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, x, y, scale, 1)
+       : sel == 2 ? __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, x, y, scale, 2)
+                  : __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, x, y, scale, 3);
+}
 __device__ __forceinline__ uint32_t cvt_fp4_4x32(u32x4 w, float scale) {  // 4 elements -> 2 bytes (low half)
   uint32_t r = 0;
   r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, as_f32(w.x), as_f32(w.y), scale, 0);

@@ -211,23 +211,49 @@ int launch_mx_fp4(const MxArgs& a) {
                                                                    a.scale);
   return launch_status();
 }
+// blocks down the columns, payload transposed: [cols, rows/2], scales [cols, rows/32]
+template <int IN, int LAYOUT>
+int launch_mx_fp4_cols(const MxArgs& a) {
+  const int64_t tiles = ceil_div(a.rows, (int64_t)kColTRows) * ceil_div(a.cols, (int64_t)kColTCols);
+  if (tiles > 0x7FFFFFFFll) return DT_ERR_INVALID_SHAPE;
+  mx_col_t_kernel<IN, DT_E2M1, LAYOUT><<<(unsigned)tiles, kBlock, 0, a.stream>>>(a.x, (uint32_t)a.rows, (uint32_t)a.cols, a.data,
+                                                                                a.scale);
+  return launch_status();
+}
 }  // namespace
 
-extern "C" int dt_mx_fp4_quantize(const void* x, int in_dtype, int64_t rows, int64_t cols, int scale_layout, void* data,
-                                  uint8_t* scale, dt_stream_t stream) {
+extern "C" int dt_mx_fp4_quantize(const void* x, int in_dtype, int64_t rows, int64_t cols, int axis, int scale_layout,
+                                  void* data, uint8_t* scale, dt_stream_t stream) {
   if (in_dtype != DT_F32 && in_dtype != DT_BF16 && in_dtype != DT_F16) return DT_ERR_INVALID_DTYPE;
+  if (axis != 0 && axis != 1) return DT_ERR_INVALID_MODE;
   if (scale_layout != DT_SCALE_PLAIN && scale_layout != DT_SCALE_BLOCKED) return DT_ERR_INVALID_MODE;
-  if (rows < 0 || cols < 0 || cols % 32 != 0) return DT_ERR_INVALID_SHAPE;
-  if (rows * cols / 32 >= (1ll << 28)) return DT_ERR_INVALID_SHAPE;  // block indices are 32 bits wide in the kernel
+  if (rows < 0 || cols < 0 || (axis == 1 ? cols : rows) % 32 != 0) return DT_ERR_INVALID_SHAPE;
   if (rows == 0 || cols == 0) return DT_OK;
   if (!x || !data || !scale) return DT_ERR_NULL_POINTER;
-  if (!dt::aligned(x, 16) || !dt::aligned(data, 4)) return DT_ERR_MISALIGNED;
   hipStream_t s = dt::as_hip(stream);
-  if (scale_layout == DT_SCALE_BLOCKED) {
+  const bool blocked = scale_layout == DT_SCALE_BLOCKED;
+  if (axis == 0) {
+    // a lane loads 4 adjacent columns of a row with one 8- or 16-byte load
+    const int64_t kB = in_dtype == DT_F32 ? 4 : 2;
+    if (cols % 4 != 0 || rows >= (1ll << 31) || cols >= (1ll << 31)) return DT_ERR_INVALID_SHAPE;
+    if (!dt::aligned(x, 4 * kB) || (cols * kB) % (4 * kB) != 0 || !dt::aligned(data, 16) || !dt::aligned(scale, 4))
+      return DT_ERR_MISALIGNED;
+    if (blocked) {
+      if (int st = zero_blocked_padding(scale, cols, rows / 32, s)) return st;
+    }
+    MxArgs a{x, rows, cols, 0, 1, static_cast<uint8_t*>(data), scale, s};
+    switch (in_dtype) {
+      case DT_F32: return blocked ? launch_mx_fp4_cols<DT_F32, DT_SCALE_BLOCKED>(a) : launch_mx_fp4_cols<DT_F32, DT_SCALE_PLAIN>(a);
+      case DT_BF16: return blocked ? launch_mx_fp4_cols<DT_BF16, DT_SCALE_BLOCKED>(a) : launch_mx_fp4_cols<DT_BF16, DT_SCALE_PLAIN>(a);
+      default: return blocked ? launch_mx_fp4_cols<DT_F16, DT_SCALE_BLOCKED>(a) : launch_mx_fp4_cols<DT_F16, DT_SCALE_PLAIN>(a);
+    }
+  }
+  if (rows * cols / 32 >= (1ll << 28)) return DT_ERR_INVALID_SHAPE;  // block indices are 32 bits wide in the kernel
+  if (!dt::aligned(x, 16) || !dt::aligned(data, 4)) return DT_ERR_MISALIGNED;
+  if (blocked) {
     if (int st = zero_blocked_padding(scale, rows, cols / 32, s)) return st;
   }
   MxArgs a{x, rows, cols, 1, 0, static_cast<uint8_t*>(data), scale, s};
-  const bool blocked = scale_layout == DT_SCALE_BLOCKED;
   switch (in_dtype) {
     case DT_F32: return blocked ? launch_mx_fp4<DT_F32, DT_SCALE_BLOCKED>(a) : launch_mx_fp4<DT_F32, DT_SCALE_PLAIN>(a);
     case DT_BF16: return blocked ? launch_mx_fp4<DT_BF16, DT_SCALE_BLOCKED>(a) : launch_mx_fp4<DT_BF16, DT_SCALE_PLAIN>(a);

@@ -367,6 +367,7 @@ __global__ __launch_bounds__(kBlock) void mx_col_kernel(const void* __restrict__
 // lane-local, and converts column by column (4 consecutive rows per packed word).  The fp8
 // bytes go to LDS as [column][128 rows] and leave as full 128-byte rows of the [cols, rows]
 // output; the 4 scale bytes of a column (one per wave) leave as one word.
+// With the e2m1 output code two rows of x share an output byte: a column's 128 rows are 64 bytes.
 constexpr int kColTRows = 128, kColTCols = 256, kColTPitch = 144;  // LDS row pitch: 128 + 16 pad
 template <int IN, int OUT, int LAYOUT>
 __global__ __launch_bounds__(kBlock) void mx_col_t_kernel(const void* __restrict__ x, uint32_t rows, uint32_t cols,
@@ -425,6 +426,25 @@ __global__ __launch_bounds__(kBlock) void mx_col_t_kernel(const void* __restrict
     for (int c = 0; c < 4; ++c) {
       const MxScale<OUT> s = mx_scale_from_absbits<OUT>(cm[c]);
       sbyte[c] = s.byte;
+      if constexpr (OUT == DT_E2M1) {
+        uint32_t r4[4];  // 8 consecutive rows per word: byte j = rows 8q+2j (low nibble), 8q+2j+1
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          uint32_t r = 0;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int i = 8 * q + 2 * j;
+            if constexpr (IN == DT_F32) {
+              r = cvt_fp4_pair32(r, word(i, c), word(i + 1, c), s.scale, j);
+            } else {
+              r = cvt_fp4_pair16<IN>(r, gather_halves(c & 1, word(i, c), word(i + 1, c)), s.scale, j);
+            }
+          }
+          r4[q] = s.nan ? 0x77777777u : r;
+        }
+        *reinterpret_cast<u32x4*>(tile + (lane * 4 + c) * kColTPitch + w * 16) = u32x4{r4[0], r4[1], r4[2], r4[3]};
+        continue;
+      }
       uint32_t r[8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) {
@@ -446,12 +466,23 @@ __global__ __launch_bounds__(kBlock) void mx_col_t_kernel(const void* __restrict
 
   // 256 output rows (columns of x) x 8 chunks of 16 bytes; 8 consecutive lanes write one row
   const uint32_t trow0 = tr * kColTRows, tcol0 = tc * kColTCols;
+  if constexpr (OUT == DT_E2M1) {  // 4 chunks of 16 bytes (32 rows of x each) per output row
 #pragma unroll
-  for (int i = 0; i < kColTCols * 8 / kBlock; ++i) {
-    const int id = tid + i * kBlock, r = id >> 3, q = id & 7;
-    if (tcol0 + r < cols && trow0 + q * 16 < rows) {
-      const u32x4 v = *reinterpret_cast<const u32x4*>(tile + r * kColTPitch + q * 16);
-      st_stream(reinterpret_cast<u32x4*>(data + (uint64_t)(tcol0 + r) * rows + trow0 + q * 16), v);
+    for (int i = 0; i < kColTCols * 4 / kBlock; ++i) {
+      const int id = tid + i * kBlock, r = id >> 2, q = id & 3;
+      if (tcol0 + r < cols && trow0 + q * 32 < rows) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(tile + r * kColTPitch + q * 16);
+        st_stream(reinterpret_cast<u32x4*>(data + (uint64_t)(tcol0 + r) * (rows / 2) + trow0 / 2 + q * 16), v);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < kColTCols * 8 / kBlock; ++i) {
+      const int id = tid + i * kBlock, r = id >> 3, q = id & 7;
+      if (tcol0 + r < cols && trow0 + q * 16 < rows) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(tile + r * kColTPitch + q * 16);
+        st_stream(reinterpret_cast<u32x4*>(data + (uint64_t)(tcol0 + r) * rows + trow0 + q * 16), v);
+      }
     }
   }
   // scales [cols, rows/32]: 4 bytes per column of this tile

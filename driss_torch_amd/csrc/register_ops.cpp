@@ -298,25 +298,30 @@ Tensor to_blocked(const Tensor& scale) {
 }
 
 // -------------------------------------------------------------------- mx_fp4_quantize
-// Operands for mx_fp4_bf16: packed e2m1 [M, N/2] (uint8, even element in the low nibble) and E8M0
-// scales per 32 elements of a row.  No counterpart op in the reference, whose GEMM test takes them
+// Operands for mx_fp4_bf16: packed e2m1 (uint8, first element of a pair in the low nibble) and E8M0
+// scales per 32 elements: axis 1 along the rows -> [M, N/2]; axis 0 down the columns, transposed ->
+// [N, M/2] (the axis-1 cast of input.t()).  No counterpart op in the reference, whose GEMM test takes them
 // from torchao's MXTensor.to_mx(x, "fp4_e2m1", 32) (test/test_mx.py:17-21).
-std::tuple<Tensor, Tensor> mx_fp4_quantize(const Tensor& input, bool blocked) {
+std::tuple<Tensor, Tensor> mx_fp4_quantize(const Tensor& input, bool blocked, int64_t axis) {
   TORCH_CHECK(input.is_cuda(), "Input tensor must be a CUDA tensor");
   TORCH_CHECK(input.is_contiguous(), "Input tensor must be contiguous");
   TORCH_CHECK(input.scalar_type() == at::kHalf || input.scalar_type() == at::kFloat ||
                   input.scalar_type() == at::kBFloat16,
               "Input tensor must be float, half, or bfloat16");
   TORCH_CHECK(input.dim() == 2, "Only support 2d tensor for now");
+  TORCH_CHECK(axis >= -2 && axis < 2, "axis must be 0 or 1");
+  const int ax = (int)((axis + 2) % 2);
   const int64_t m = input.size(0), n = input.size(1);
-  TORCH_CHECK(n % 32 == 0, "Need block shape to evenly divide the input tensor for now");
+  const int64_t outer = ax == 1 ? m : n, inner = ax == 1 ? n : m;  // payload [outer, inner / 2]
+  TORCH_CHECK(inner % 32 == 0, "Need block shape to evenly divide the input tensor for now");
+  TORCH_CHECK(ax == 1 || n % 4 == 0, "The column-wise cast needs a multiple of 4 columns");
   Ctx ctx(input);
-  Tensor data = at::empty({m, n / 2}, input.options().dtype(at::kByte));
-  Tensor scale = at::empty({blocked ? dt_blocked_scale_bytes(m, n / 32) : m * (n / 32)},
+  Tensor data = at::empty({outer, inner / 2}, input.options().dtype(at::kByte));
+  Tensor scale = at::empty({blocked ? dt_blocked_scale_bytes(outer, inner / 32) : outer * (inner / 32)},
                            input.options().dtype(at::kFloat8_e8m0fnu));
   if (input.numel() == 0) return {data, scale};
   TORCH_CHECK(reinterpret_cast<std::uintptr_t>(input.data_ptr()) % 16 == 0, "Input tensor must be 16-byte aligned");
-  check_status(dt_mx_fp4_quantize(input.data_ptr(), in_code(input), m, n, blocked ? DT_SCALE_BLOCKED : DT_SCALE_PLAIN,
+  check_status(dt_mx_fp4_quantize(input.data_ptr(), in_code(input), m, n, ax, blocked ? DT_SCALE_BLOCKED : DT_SCALE_PLAIN,
                                   data.data_ptr(), static_cast<uint8_t*>(scale.data_ptr()), ctx.stream),
                "mx_fp4_quantize");
   return {data, scale};
@@ -451,7 +456,7 @@ TORCH_LIBRARY(DrissTorch, m) {
   m.impl("mx_fp8_quantize_ex", c10::DispatchKey::CUDA, TORCH_FN(driss_torch::mx_fp8_quantize_ex));
   m.def("mx_fp8_quantize_dual(Tensor input, ScalarType fp8_type, bool blocked) -> (Tensor, Tensor, Tensor, Tensor)");
   m.impl("mx_fp8_quantize_dual", c10::DispatchKey::CUDA, TORCH_FN(driss_torch::mx_fp8_quantize_dual));
-  m.def("mx_fp4_quantize(Tensor input, bool blocked) -> (Tensor, Tensor)");
+  m.def("mx_fp4_quantize(Tensor input, bool blocked, int axis) -> (Tensor, Tensor)");
   m.impl("mx_fp4_quantize", c10::DispatchKey::CUDA, TORCH_FN(driss_torch::mx_fp4_quantize));
   m.def("to_blocked(Tensor scale) -> Tensor");
   m.impl("to_blocked", c10::DispatchKey::CUDA, TORCH_FN(driss_torch::to_blocked));

@@ -191,15 +191,19 @@ DT_API int dt_mx_fp4_bf16(const void* a, const void* b, const uint8_t* sfa, cons
                           int64_t ldo, dt_stream_t stream);
 
 /* ------------------------------------------------------------------ mx_fp4_quantize --
- * MXFP4 operands for dt_mx_fp4_bf16: x [rows, cols] -> e2m1 pairs [rows, cols/2] (even element in
- * the low nibble) and one E8M0 byte per 32 elements along a row, plain [rows, cols/32] or blocked.
- * The reference has no such op: its GEMM test takes the operands from torchao's
- * MXTensor.to_mx(x, "fp4_e2m1", 32) (test/test_mx.py:17-21), whose default scale is restated
- * here: shared exponent floor(log2(max|x|)) - 2 from the fp32 exponent field, clamped to
- * [-127, 127]; payload = e2m1_rne_saturating(x * 2^-exponent).  A zero block gives byte 0; a block
- * that holds a NaN gives byte 255 and 0x7 in every nibble; an infinite maximum gives byte 253.
- * cols % 32 == 0, x 16-byte aligned, data 4-byte aligned, rows * cols < 2^33.              */
-DT_API int dt_mx_fp4_quantize(const void* x, int in_dtype, int64_t rows, int64_t cols,
+ * MXFP4 operands for dt_mx_fp4_bf16: e2m1 pairs (first element of a pair in the low nibble) and one
+ * E8M0 byte per 32 elements.  axis 1: blocks along the rows of x [rows, cols] -> payload
+ * [rows, cols/2], scales [rows, cols/32]; axis 0: blocks down the columns, payload transposed ->
+ * [cols, rows/2] (pairs of adjacent rows of x), scales [cols, rows/32], i.e. the axis-1 cast of x^T.
+ * Scales plain (row-major) or blocked.  The reference has no such op: its GEMM test takes the
+ * operands from torchao's MXTensor.to_mx(x, "fp4_e2m1", 32) (test/test_mx.py:17-21), whose default
+ * scale is restated here: shared exponent floor(log2(max|x|)) - 2 from the fp32 exponent field,
+ * clamped to [-127, 127]; payload = e2m1_rne_saturating(x * 2^-exponent).  A zero block gives byte
+ * 0; a block that holds a NaN gives byte 255 and 0x7 in every nibble; an infinite maximum gives
+ * byte 253.  The blocked dimension % 32 == 0.  axis 1: x 16-byte aligned, data 4-byte aligned,
+ * rows * cols < 2^33; axis 0: cols % 4 == 0, x aligned to 4 elements, data 16-byte and scale
+ * 4-byte aligned.                                                                          */
+DT_API int dt_mx_fp4_quantize(const void* x, int in_dtype, int64_t rows, int64_t cols, int axis,
                               int scale_layout, void* data, uint8_t* scale, dt_stream_t stream);
 
 /* ------------------------------------------------- block-scaled GEMM with a workspace --

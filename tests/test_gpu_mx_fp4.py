@@ -218,6 +218,27 @@ def test_mx_fp4_cast_against_oracle(d, in_dtype, shape):
     _check_fp4_cast(d, x.to(in_dtype))
 
 
+def _check_fp4_cast_cols(d, x):
+    """blocks down the columns, payload transposed: the row-wise cast of x^T"""
+    M, N = x.shape
+    rd, rs = co.mx_fp4_quantize(x.t().contiguous())
+    for blocked in (False, True):
+        data, scale = d.mx_fp4_quantize(x.cuda(), blocked, 0)
+        assert data.shape == (N, M // 2) and torch.equal(data.cpu(), rd)
+        assert torch.equal(util.codes(scale), (co.to_blocked(rs) if blocked else rs).flatten())
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("shape", [(32, 128), (64, 4), (96, 76), (256, 512), (1024, 384), (160, 1028), (4096, 2048)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+def test_mx_fp4_cast_down_the_columns(d, in_dtype, shape):
+    g = util.gen(shape[0] * 3 + shape[1])
+    x = torch.randn(shape, generator=g) * torch.exp(2.0 * torch.randn(shape, generator=g))
+    if in_dtype == torch.float16:
+        x = x.clamp(-6.0e4, 6.0e4)
+    _check_fp4_cast_cols(d, x.to(in_dtype))
+
+
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
 def test_mx_fp4_cast_special_blocks(d, in_dtype):
     x = util.normal((128, 512), 41, in_dtype)
@@ -234,6 +255,7 @@ def test_mx_fp4_cast_special_blocks(d, in_dtype):
     x[8, :32] = (torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0] * 4)).to(in_dtype)   # the grid's ties
     x[9, :32] = -x[8, :32]
     _check_fp4_cast(d, x)
+    _check_fp4_cast_cols(d, x.t().contiguous())
 
 
 def test_mx_fp4_cast_every_bf16_pattern(d):
@@ -250,6 +272,7 @@ def test_mx_fp4_cast_every_bf16_pattern(d):
     rows.append(pats.float().view(64, 1024))  # with NaN and infinity patterns in place
     x = torch.cat(rows).to(torch.bfloat16)
     _check_fp4_cast(d, x)
+    _check_fp4_cast_cols(d, x.t().contiguous())
 
 
 def test_mx_fp4_cast_feeds_the_gemm(d):
@@ -283,9 +306,14 @@ def test_mx_fp4_cast_errors_and_compile(d, cabi):
     L = cabi.lib()
     data = torch.empty(64 * 64 + 8, dtype=torch.uint8, device="cuda")
     scale = torch.empty(64 * 4, dtype=torch.uint8, device="cuda")
-    assert L.dt_mx_fp4_quantize(x.data_ptr(), cabi.BF16, 64, 128, 0, data.data_ptr() + 2, scale.data_ptr(), None) == 4
-    assert L.dt_mx_fp4_quantize(x.data_ptr(), cabi.BF16, 64, 128, 2, data.data_ptr(), scale.data_ptr(), None) == 6
-    assert L.dt_mx_fp4_quantize(x.data_ptr(), 7, 64, 128, 0, data.data_ptr(), scale.data_ptr(), None) == 1
+    assert L.dt_mx_fp4_quantize(x.data_ptr(), cabi.BF16, 64, 128, 1, 0, data.data_ptr() + 2, scale.data_ptr(), None) == 4
+    assert L.dt_mx_fp4_quantize(x.data_ptr(), cabi.BF16, 64, 128, 1, 2, data.data_ptr(), scale.data_ptr(), None) == 6
+    assert L.dt_mx_fp4_quantize(x.data_ptr(), cabi.BF16, 64, 128, 3, 0, data.data_ptr(), scale.data_ptr(), None) == 6
+    assert L.dt_mx_fp4_quantize(x.data_ptr(), 7, 64, 128, 1, 0, data.data_ptr(), scale.data_ptr(), None) == 1
+    assert L.dt_mx_fp4_quantize(x.data_ptr(), cabi.BF16, 48, 128, 0, 0, data.data_ptr(), scale.data_ptr(), None) == 2  # 48 rows down the columns
+    assert L.dt_mx_fp4_quantize(x.data_ptr(), cabi.BF16, 64, 128, 0, 0, data.data_ptr() + 4, scale.data_ptr(), None) == 4
+    with pytest.raises(RuntimeError):
+        d.mx_fp4_quantize(x[:48].contiguous(), False, 0)
     fn = torch.compile(lambda t: d.mx_fp4_quantize(t, True), fullgraph=True, backend="aot_eager")
     got, want = fn(x), d.mx_fp4_quantize(x, True)
     assert torch.equal(got[0], want[0]) and torch.equal(util.codes(got[1]), util.codes(want[1]))

@@ -70,6 +70,11 @@ def test_mx_casts_random_shapes(d, shape, in_dtype):
         for blocked in (False, True):
             data, scale = d.mx_fp4_quantize(g, blocked)
             assert torch.equal(data.cpu(), fd) and torch.equal(util.codes(scale), (co.to_blocked(fs) if blocked else fs).flatten())
+    if rows % 32 == 0 and cols % 4 == 0:  # ... and down the columns (the cast of x^T)
+        fd, fs = co.mx_fp4_quantize(x.t().contiguous())
+        for blocked in (False, True):
+            data, scale = d.mx_fp4_quantize(g, blocked, 0)
+            assert torch.equal(data.cpu(), fd) and torch.equal(util.codes(scale), (co.to_blocked(fs) if blocked else fs).flatten())
     for fp8 in (E4, E5):
         if cols % 32 == 0:
             rd, rs = co.mx_quantize(x, axis=1, transpose=False, out_dtype=fp8)
