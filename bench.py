@@ -150,7 +150,7 @@ def main():
     cabi.set_tuning("dynamic.resident", 1)
 
     result = {
-        "metric": "cast/amax HBM GB/s (% of 8 TB/s) at 8192^2 bf16; MXFP8 GEMM TFLOPS",
+        "metric": "cast/amax HBM GB/s (% of 8 TB/s) at 8192² bf16; MXFP8 GEMM TFLOPS",
         "value": round(value, 1),
         "unit": "GB/s",
         "n_gpus": 1,
