@@ -5,6 +5,7 @@ test/test_sat_cast.py:45-62, which does this for saturated_cast only."""
 import pytest
 import torch
 
+from oracle import eager
 from tests import util
 
 pytestmark = pytest.mark.gpu
@@ -83,6 +84,32 @@ def test_mx_quantize_blocked_and_gemm_compile(d):
 def test_to_blocked_compile(d):
     s = torch.randint(0, 255, (256, 12), dtype=torch.uint8, device="cuda")
     _same(_compiled(d.to_blocked)(s), d.to_blocked(s))
+
+
+@pytest.mark.parametrize("fp8_dtype", [E4, E5])
+def test_saturated_cast_compile_default_backend(d, fp8_dtype):
+    """test/test_sat_cast.py:45-62 as written there: torch.compile with its default backend"""
+    torch._dynamo.reset()
+    a = util.uniform((64, 512), 95).cuda()
+    scale = eager.tensor_to_scale(a, fp8_dtype)
+    fn = torch.compile(d.saturated_cast, fullgraph=True)
+    _same(fn(a, scale, fp8_dtype), d.saturated_cast(a, scale, fp8_dtype))
+
+
+def test_quantize_gemm_step_compile_default_backend(d):
+    """a compiled function that mixes the ops with ordinary tensor code (generated kernels before and
+    after the custom calls): per-tensor quantization, both MX casts, the GEMM"""
+    torch._dynamo.reset()
+
+    def step(a, w):
+        q, amax, scale = d.dynamic_scaled_quant_ex(a * 0.5, E4, 0)
+        qa, sa = d.mx_fp8_quantize_blocked(a + 1.0)
+        qw, sw = d.mx_fp8_quantize_blocked(w)
+        y = d.mx_fp8_bf16(qa, qw.t(), sa, sw)
+        return y * 2.0 + amax.to(torch.bfloat16), q, scale
+
+    a, w = util.normal((256, 512), 96).cuda(), util.normal((384, 512), 97).cuda()
+    _same(torch.compile(step, fullgraph=True)(a, w), step(a, w))
 
 
 def test_ops_replay_from_a_captured_graph(d):
