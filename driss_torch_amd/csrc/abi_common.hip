@@ -1,6 +1,7 @@
 // Status strings, device facts, tuning knobs and the workspace entry points of the C ABI.
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "dt_device.hpp"
@@ -11,7 +12,7 @@ namespace dt {
 namespace {
 struct Knob {
   const char* key;
-  int value;
+  std::atomic<int> value;  // set from any thread while launches on other threads read it
 };
 // Launch-shape knobs.  Workgroups per CU for the persistent grids, chosen on MI355X.
 //   dynamic.resident: 1 = per-tensor dynamic quantization of a tensor that fits the chip runs as one
@@ -55,7 +56,7 @@ std::once_flag g_facts_once[kMaxDevices];
 
 int tuning(const char* key) {
   for (int i = 0; i < kNumKnobs; ++i)
-    if (strcmp(g_knobs[i].key, key) == 0) return g_knobs[i].value;
+    if (strcmp(g_knobs[i].key, key) == 0) return g_knobs[i].value.load(std::memory_order_relaxed);
   return 0;
 }
 
@@ -112,7 +113,7 @@ int dt_set_tuning(const char* key, int value) {
   if (!key) return DT_ERR_NULL_POINTER;
   for (int i = 0; i < dt::kNumKnobs; ++i)
     if (strcmp(dt::g_knobs[i].key, key) == 0) {
-      dt::g_knobs[i].value = value;
+      dt::g_knobs[i].value.store(value, std::memory_order_relaxed);
       return DT_OK;
     }
   return DT_ERR_INVALID_MODE;
@@ -122,7 +123,7 @@ int dt_get_tuning(const char* key, int* value) {
   if (!key || !value) return DT_ERR_NULL_POINTER;
   for (int i = 0; i < dt::kNumKnobs; ++i)
     if (strcmp(dt::g_knobs[i].key, key) == 0) {
-      *value = dt::g_knobs[i].value;
+      *value = dt::g_knobs[i].value.load(std::memory_order_relaxed);
       return DT_OK;
     }
   return DT_ERR_INVALID_MODE;

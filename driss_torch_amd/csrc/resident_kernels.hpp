@@ -19,6 +19,8 @@
 // end of the kernel whatever happens.
 #pragma once
 
+#include <atomic>
+
 #include <mutex>
 
 #include "quant_kernels.hpp"
@@ -284,14 +286,14 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
   if (dev < 0 || dev >= ResidentGate::kMaxDevices) return kResidentNotTaken;
   // per instantiation and device (a function's attributes live with the device's copy of the code);
   // the call is idempotent, so a race between threads only repeats it
-  static bool configured[ResidentGate::kMaxDevices] = {};
-  if (!configured[dev]) {
+  static std::atomic<bool> configured[ResidentGate::kMaxDevices] = {};
+  if (!configured[dev].load(std::memory_order_relaxed)) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)kResLdsBytes) != hipSuccess) {
       (void)hipGetLastError();
       return kResidentNotTaken;
     }
-    configured[dev] = true;
+    configured[dev].store(true, std::memory_order_relaxed);
   }
   uint8_t* w = static_cast<uint8_t*>(ws);
   uint8_t* o = static_cast<uint8_t*>(out);
