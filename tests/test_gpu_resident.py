@@ -141,6 +141,37 @@ def test_resident_back_to_back_and_two_streams(cabi):
             assert int(ws[196:200].cpu().view(torch.int32).item()) == 0
 
 
+def test_resident_not_taken_on_a_stream_restricted_to_some_cus(cabi):
+    """a stream created with a CU mask of half the chip could never hold one workgroup per CU at
+    once: the library sees the mask and takes the two kernels there (right results, no give-up flag;
+    the spin limit is lowered so that a launch of the resident kernel would show up at once)"""
+    import ctypes
+
+    hip = ctypes.CDLL("libamdhip64.so")
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    words = (cus + 31) // 32
+    mask = (ctypes.c_uint32 * words)(*([0xFFFFFFFF] * (words // 2) + [0] * (words - words // 2)))
+    handle = ctypes.c_void_p()
+    assert hip.hipExtStreamCreateWithCUMask(ctypes.byref(handle), ctypes.c_uint32(words), mask) == 0
+    stream = torch.cuda.ExternalStream(handle.value)
+    cabi.set_tuning("dynamic.resident", 1)
+    cabi.set_tuning("dynamic.resident_spin_limit", 64)
+    x = util.normal_with_outliers((4096, 4096), 77)
+    xg = x.cuda()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        o4, o5, amax, scales = cabi.dynamic_scaled_quant_pair(xg, 2)
+        flag_ws = cabi.workspace(torch.device("cuda"))
+        small = cabi.dynamic_scaled_quant(xg[:8], E4, 2)  # a grid of few workgroups fits the masked CUs: resident
+    stream.synchronize()
+    r4, ramax, _ = co.dynamic_scaled_quant(x, E4, co.ROUND_V2)
+    r5, _, _ = co.dynamic_scaled_quant(x, E5, co.ROUND_V2)
+    assert torch.equal(util.codes(o4), r4) and torch.equal(util.codes(o5), r5) and amax.item() == ramax.item()
+    assert torch.equal(util.codes(small[0]), co.dynamic_scaled_quant(x[:8], E4, co.ROUND_V2)[0])
+    assert int(flag_ws[196:200].cpu().view(torch.int32).item()) == 0
+    cabi.set_tuning("dynamic.resident_spin_limit", 1 << 19)
+
+
 def test_resident_wait_gives_up_loudly(cabi):
     """with a spin limit of one poll most workgroups stop waiting before the last one has arrived:
     every wave still runs to the end, the sticky flag is set and those workgroups write NaN"""
