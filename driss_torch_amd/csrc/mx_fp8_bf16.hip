@@ -548,6 +548,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   constexpr int kRowsPerPass = kWave / kChunksPerRow;    // rows one store instruction covers
   const int erow = lane / kChunksPerRow, echunk = lane % kChunksPerRow;
   const int n = n0 + wn * WN + echunk * 8;
+  // a tile wholly inside the matrix with an aligned output (the common case): no edge tests, the
+  // row pointer moves by a constant
+  if (wide_stores && m0 + BM <= M && n0 + BN <= N) {
+    uint16_t* dst = out + (int64_t)(m0 + wm * WM + erow) * ldo + n;
+    const int64_t pass_stride = (int64_t)kRowsPerPass * ldo;
+    const uint8_t* src = epi + erow * kEpiPitch + echunk * 16;
+#pragma unroll
+    for (int r = 0; r < WM; r += kRowsPerPass) {
+      *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(src + r * kEpiPitch);
+      dst += pass_stride;
+    }
+    return;
+  }
 #pragma unroll
   for (int r = 0; r < WM; r += kRowsPerPass) {
     const int row = r + erow;
