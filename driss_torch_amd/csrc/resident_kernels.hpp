@@ -293,9 +293,6 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
   int64_t grid = ceil_div(nvec, (int64_t)kBlock * 4);  // at least 4 vectors per lane before another workgroup joins
   if (grid > cus) grid = cus;
   if (grid < 1) grid = 1;
-  // every workgroup waits for all the others: a stream that may not use as many CUs as the grid has
-  // workgroups could never hold them all at once
-  if (stream_cu_count(stream) < grid) return kResidentNotTaken;
   auto kernel = resident_quant_kernel<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR>;
   int dev = 0;
   (void)hipGetDevice(&dev);
@@ -325,6 +322,9 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
     (void)hipGetLastError();
     return kResidentNotTaken;
   }
+  // every workgroup waits for all the others: a stream that may not use as many CUs as the grid has
+  // workgroups could never hold them all at once
+  if (stream_cu_count(stream) < grid) return kResidentNotTaken;
   if (gate.used[dev] && gate.last_stream[dev] != stream) {
     // mark the tail of the stream that ran the previous resident kernel and wait for it here
     if (!gate.event[dev] && hipEventCreateWithFlags(&gate.event[dev], hipEventDisableTiming) != hipSuccess) {
