@@ -250,6 +250,43 @@ def test_mx_gemm_strided_operands_and_output(d, cabi, size):
     assert (out_wide[:, :8] == 7.0).all() and (out_wide[:, 8 + N:] == 7.0).all()  # nothing written outside
 
 
+def _random_plan_sizes(seed, n):
+    import random
+
+    rng = random.Random(seed)
+    return [(rng.randint(1, 6000), 128 * rng.randint(1, 3), 8 * rng.randint(1, 750)) for _ in range(n)]
+
+
+@pytest.mark.parametrize("size", _random_plan_sizes(11, 10), ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+def test_mx_gemm_random_sizes_across_launch_plans(d, size):
+    """random (M, K, N) up to 6000 x 6000 outputs, ragged in both directions: whichever plan the
+    library picks (small tiles, 256 x 128 tiles, whole rounds of big tiles with the leftover as
+    quadrants or halves), every entry is within the tolerance of the fp32 product of the
+    dequantized operands (computed on the device: a library matmul is the reference here)"""
+    M, K, N = size
+    g = torch.Generator(device="cuda").manual_seed(M * 7 + N)
+    a = torch.randn((M, K), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    b = torch.randn((N, K), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    a_data, a_scale = d.mx_fp8_quantize(a)
+    b_data, b_scale = d.mx_fp8_quantize(b)
+    out = d.mx_fp8_bf16(a_data, b_data.t(), d.to_blocked(a_scale.view(M, K // 32)), d.to_blocked(b_scale.view(N, K // 32)))
+
+    def dequant(data, scale, rows):
+        s = torch.exp2(scale.view(torch.uint8).view(rows, K // 32).float() - 127.0).repeat_interleave(32, dim=1)
+        return data.float() * s
+
+    da, db = dequant(a_data, a_scale, M), dequant(b_data, b_scale, N)
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        ref = da @ db.T
+        bound = da.abs() @ db.abs().T
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+    err = (out.float() - ref).abs()
+    assert bool((err <= bound * 2**-8 + 1e-30).all()), f"max rel {(err / bound).max().item():.3e}"
+
+
 def test_mx_gemm_split_k_on_two_streams(d):
     """split-K products issued alternately on two streams (each stream has its own ticket counters and
     parking space in the torch shim): every result equals the one computed alone"""
