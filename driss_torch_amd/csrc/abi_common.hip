@@ -18,6 +18,8 @@ struct Knob {
 //   dynamic.resident: 1 = per-tensor dynamic quantization of a tensor that fits the chip runs as one
 //                 kernel that keeps it in registers and LDS; dynamic.resident_min_kib = smallest such
 //                 tensor; sizes in [resident_gap_lo_kib, resident_gap_hi_kib) take the two kernels
+//                 dynamic.resident_overflow: 1 = tensors of up to 4 x the chip's capacity keep what fits
+//                 and read only the rest twice
 //   mx.dual:      1 = dt_mx_fp8_quantize_dual reads x once (0: two single casts)
 //   mx.colt_via_dual: 1 = the transposed column cast runs as the one-read kernel without its row half
 //   mx.row_band4: 1 = row-wise MX cast with blocked scales walks 4 rows x 512 elements per wave pass
@@ -45,6 +47,7 @@ Knob g_knobs[] = {
     {"dynamic.resident_min_kib", 0},
     {"dynamic.resident_gap_lo_kib", 12288},
     {"dynamic.resident_gap_hi_kib", 40960},
+    {"dynamic.resident_overflow", 1},
     {"dynamic.resident_spin_limit", 1 << 19},
 };
 constexpr int kNumKnobs = sizeof(g_knobs) / sizeof(g_knobs[0]);

@@ -57,7 +57,12 @@ __device__ __forceinline__ void cast_vec_pair_finite(u32x4 w, float s4, uint8_t*
   }
 }
 
-template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR>
+// OVERFLOW: the tensor is larger than the chip holds (up to kResMaxOver times).  A workgroup's
+// share then has vector slots past the kResVecs it can keep: pass 1 streams those first (reduce
+// only), pass 2 reads them again after the kept part has been converted.  Memory sees the kept
+// part once and only the rest twice.
+constexpr int kResMaxOver = 4;
+template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR, bool OVERFLOW = false>
 __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __restrict__ x, int64_t nvec, int tail,
                                                                uint8_t* __restrict__ ws, uint8_t* __restrict__ out,
                                                                uint8_t* __restrict__ out2, float* __restrict__ amax_out,
@@ -101,6 +106,17 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
   // the chip's capacity skips whole batches (a branch the workgroup takes as one), in both passes.
   const uint32_t block_first = blockIdx.x * kBlock;
   const uint32_t nk = block_first < (uint32_t)nvec ? ((uint32_t)nvec - block_first + (uint32_t)stride - 1u) / (uint32_t)stride : 0u;
+  if constexpr (OVERFLOW) {  // slots that cannot be kept: before anything is held in registers
+    for (uint32_t k0 = kResVecs; k0 < nk; k0 += kResBatch) {
+      u32x4 t[kResBatch];
+#pragma unroll
+      for (int j = 0; j < kResBatch; ++j) t[j] = fetch((int)k0 + j);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < kResBatch; ++j) absorb((int)k0 + j, t[j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
   // the LDS part first (through a batch of registers), then the register part in place
 #pragma unroll
   for (int b = 0; b < kResLdsVecs; b += kResBatch) {
@@ -241,6 +257,20 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
       for (int j = 0; j < kResBatch; ++j)
         if (b + j < kResLdsVecs) emit(kResRegVecs + b + j, keep[(b + j) * kBlock + tid]);
     }
+    if constexpr (OVERFLOW) {  // the slots that were not kept: read again, the registers are free now
+      for (uint32_t k0 = kResVecs; k0 < nk; k0 += kResBatch) {
+        u32x4 t[kResBatch];
+#pragma unroll
+        for (int j = 0; j < kResBatch; ++j) {
+          const uint32_t i = first2 + (k0 + j) * stride32;
+          t[j] = ld_stream(v + (i < nvec32 ? i : nvec32 - 1u));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < kResBatch; ++j) emit((int)k0 + j, t[j]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
   }
   if (blockIdx.x == 0 && tid < tail) {
     const int64_t e = nvec * kV + tid;
@@ -278,7 +308,7 @@ inline int stream_cu_count(hipStream_t stream) {
 // Launch the resident kernel if the tensor qualifies.  Returns DT_OK when it was launched, a
 // negative value when the caller should take the two-kernel path instead.
 constexpr int kResidentNotTaken = -1;
-template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR>
+template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR, bool OVERFLOW = false>
 inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* out, void* out2, float* amax_out,
                                 float* scale_out, float fmax0, float fmax1, hipStream_t stream) {
   if constexpr (PAIR && OUT != DT_E4M3FN) return kResidentNotTaken;  // the pair is (e4m3fn, e5m2)
@@ -289,11 +319,17 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
   const int cus = device_facts().cu_count;
   int64_t nvec = numel / kV;
   int tail = (int)(numel % kV);
-  if (nvec < 1 || nvec > (int64_t)cus * kBlock * kResVecs) return kResidentNotTaken;
+  const int64_t capacity = (int64_t)cus * kBlock * kResVecs;
+  if constexpr (!OVERFLOW) {
+    if (nvec > capacity && nvec <= capacity * kResMaxOver && tuning("dynamic.resident_overflow"))
+      return launch_resident_impl<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR, true>(x, numel, ws, out, out2, amax_out, scale_out,
+                                                                                fmax0, fmax1, stream);
+  }
+  if (nvec < 1 || nvec > capacity * (OVERFLOW ? kResMaxOver : 1)) return kResidentNotTaken;
   int64_t grid = ceil_div(nvec, (int64_t)kBlock * 4);  // at least 4 vectors per lane before another workgroup joins
   if (grid > cus) grid = cus;
   if (grid < 1) grid = 1;
-  auto kernel = resident_quant_kernel<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR>;
+  auto kernel = resident_quant_kernel<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR, OVERFLOW>;
   int dev = 0;
   (void)hipGetDevice(&dev);
   if (dev < 0 || dev >= ResidentGate::kMaxDevices) return kResidentNotTaken;

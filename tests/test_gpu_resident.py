@@ -100,8 +100,8 @@ def test_resident_special_values(cabi, in_dtype):
 
 
 def test_resident_capacity_boundary(cabi):
-    """8192 x 8192 bf16 (and 8192 x 4096 fp32) is exactly what 256 CUs hold; one more row does not
-    fit and goes through the two kernels"""
+    """8192 x 8192 bf16 (and 8192 x 4096 fp32) is exactly what 256 CUs hold; with one more row the
+    kernel keeps what fits and reads the rest twice"""
     cabi.set_tuning("dynamic.resident", 1)
     for shape, dtype in (((8192, 8192), torch.bfloat16), ((8192, 4096), torch.float32), ((8193, 8192), torch.bfloat16)):
         x = util.normal_with_outliers(shape, 1002, dtype)
@@ -111,6 +111,55 @@ def test_resident_capacity_boundary(cabi):
         r5, _, rs5 = co.dynamic_scaled_quant(x, E5, mode)
         assert torch.equal(util.codes(o4), r4) and torch.equal(util.codes(o5), r5)
         assert amax.item() == ramax.item() and scales.tolist() == [rs4.item(), rs5.item()]
+    assert _timeout_flag(cabi) == 0
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
+def test_resident_with_overflow_against_oracle(cabi, in_dtype):
+    """a tensor somewhat larger than the chip holds, ragged, with the maximum in the part that is not
+    kept (the slots past the 128th of a lane's share) and in the kept part: oracle, every rounding mode"""
+    cabi.set_tuning("dynamic.resident", 1)
+    cols = 8200 if in_dtype == torch.bfloat16 else 4100
+    x = util.normal_with_outliers((9001, cols), 1003, in_dtype)
+    modes = (1, 2, 3) if in_dtype == torch.bfloat16 else (3,)
+    for where in ((9000, cols - 3), (17, 5)):
+        x[where] = 16384.0
+        g = x.cuda()
+        for mode in modes:
+            out, amax, scale = cabi.dynamic_scaled_quant(g, E5, mode)
+            ref, ramax, rscale = co.dynamic_scaled_quant(x, E5, getattr(co, MODE[mode]))
+            assert amax.item() == ramax.item() == 16384.0 and scale.item() == rscale.item()
+            assert torch.equal(util.codes(out), ref)
+        o4, o5, amax, scales = cabi.dynamic_scaled_quant_pair(g, modes[-1])
+        r4, _, rs4 = co.dynamic_scaled_quant(x, E4, getattr(co, MODE[modes[-1]]))
+        assert torch.equal(util.codes(o4), r4) and scales[0].item() == rs4.item()
+        x[where] = 0.5
+    assert _timeout_flag(cabi) == 0
+
+
+def test_resident_with_overflow_sizes_and_special_values(cabi):
+    """from one vector past the capacity to four times the capacity (and just beyond, where the two
+    kernels take over): the same bits as the two-kernel path, also with an infinity or a NaN in the
+    part that is read twice"""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    cap = cus * 256 * 128 * 8  # bf16 elements the chip holds
+    base = util.normal_with_outliers((1, 1 << 20), 1004, torch.bfloat16).cuda()
+    for numel in (cap + 8, cap + 8 * 256 * cus + 3, 2 * cap - 5, 4 * cap, 4 * cap + 8):
+        x = base.repeat(1, numel // base.numel() + 1)[:, :numel].contiguous()
+        x[0, numel - 7] = 768.0
+        for special in (None, float("inf"), float("nan")):
+            if special is not None:
+                x[0, numel - 100] = special
+            cabi.set_tuning("dynamic.resident_overflow", 1)
+            a = cabi.dynamic_scaled_quant_pair(x, 2)
+            cabi.set_tuning("dynamic.resident_overflow", 0)
+            b = cabi.dynamic_scaled_quant_pair(x, 2)
+            cabi.set_tuning("dynamic.resident_overflow", 1)
+            assert torch.equal(util.codes(a[0]), util.codes(b[0])) and torch.equal(util.codes(a[1]), util.codes(b[1]))
+            assert torch.equal(a[2].view(torch.int32), b[2].view(torch.int32)) and torch.equal(a[3].view(torch.int32), b[3].view(torch.int32))
+            if special is None:
+                assert a[2].item() == 768.0
+        del x
     assert _timeout_flag(cabi) == 0
 
 
