@@ -245,6 +245,12 @@ def extra_kernels(torch, cabi, util, dev, K, W, gemm_only=False):
                 lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
                            torch.empty(1, device=dev), torch.empty(1, device=dev)),
                 lambda x, o, a, s_: cabi.dynamic_scaled_quant(x, e4, cabi.ROUND_BF16_SCALE_PRODUCT, o, a, s_))
+        # twice what the chip holds: 128 MiB stays in registers and LDS, the other 128 MiB is read twice
+        n2 = 16384 * 8192
+        hbm_row("dynamic_scaled_quant pair, 2 x the chip's capacity", "bf16 [16384,8192] -> amax, scales, e4m3fn and e5m2", n2 * 6,
+                lambda i: (rnd((16384, 8192), bf16, i), torch.empty((16384, 8192), dtype=e4, device=dev),
+                           torch.empty((16384, 8192), dtype=e5, device=dev), torch.empty(1, device=dev), torch.empty(2, device=dev)),
+                lambda x, o4, o5, a, s_: cabi.dynamic_scaled_quant_pair(x, cabi.ROUND_BF16_SCALE_PRODUCT, o4, o5, a, s_))
         nr = 16384 * 4096
         for dt_, nm, b in ((f32, "fp32", 4), (bf16, "bf16", 2)):
             hbm_row("dynamic_scaled_quant_rowwise", f"config 3: {nm} [16384,4096] -> e4m3fn", nr * (b + 1) + 16384 * 8,
