@@ -20,6 +20,8 @@ struct Knob {
 //                 tensor; sizes in [resident_gap_lo_kib, resident_gap_hi_kib) take the two kernels
 //                 dynamic.resident_overflow: 1 = tensors of up to 4 x the chip's capacity keep what fits
 //                 and read only the rest twice
+//   rowwise.block_from_vecs: rows of at least this many 16-byte vectors get a workgroup each (shorter
+//                 ones a wave each)
 //   mx.dual:      1 = dt_mx_fp8_quantize_dual reads x once (0: two single casts)
 //   mx.colt_via_dual: 1 = the transposed column cast runs as the one-read kernel without its row half
 //   mx.row_band4: 1 = row-wise MX cast with blocked scales walks 4 rows x 512 elements per wave pass
@@ -35,6 +37,7 @@ Knob g_knobs[] = {
     {"amax.stream_before_cast", 0},
     {"cast.blocks_per_cu", 2},
     {"cast.pair_blocks_per_cu", 2},
+    {"rowwise.block_from_vecs", 257},
     {"mx.blocks_per_cu", 32},
     {"mx.col_blocks_per_cu", 32},
     {"mx.dual", 1},

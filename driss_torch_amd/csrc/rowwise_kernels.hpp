@@ -55,6 +55,51 @@ __global__ __launch_bounds__(kBlock) void rowwise_wave_kernel(const void* __rest
   }
 }
 
+// Longer rows: one workgroup per row, NV vectors per lane kept in registers between the reduction
+// (one LDS exchange between the four waves) and the cast: still a single read of the row.
+template <int IN, int OUT, int NV>
+__global__ __launch_bounds__(kBlock) void rowwise_block_resident_kernel(const void* __restrict__ x, int row_vecs,
+                                                                        uint8_t* __restrict__ out,
+                                                                        float* __restrict__ amax_out,
+                                                                        float* __restrict__ scale_out) {
+  constexpr int kV = InTraits<IN>::kVec;
+  saturate_fp8_conversions();
+  __shared__ uint32_t lds[kBlock / kWave];
+  const int tid = threadIdx.x;
+  const int64_t row = blockIdx.x;
+  const u32x4* v = static_cast<const u32x4*>(x) + row * row_vecs;
+  u32x4 w[NV];
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int j = tid + u * kBlock;
+    w[u] = j < row_vecs ? ld_stream(v + j) : u32x4{0u, 0u, 0u, 0u};
+  }
+  uint32_t m = 0;
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    if constexpr (IN == DT_F32) {
+      m = umax(m, umax(umax(absbits_f32(w[u].x), absbits_f32(w[u].y)), umax(absbits_f32(w[u].z), absbits_f32(w[u].w))));
+    } else {
+      m = pk_absmax16(pk_absmax16(m, w[u].x), w[u].y);
+      m = pk_absmax16(pk_absmax16(m, w[u].z), w[u].w);
+    }
+  }
+  if constexpr (IN != DT_F32) m = umax(m & 0xFFFFu, m >> 16) << 16;
+  m = block_umax<kBlock / kWave>(m, lds);
+  const float amax = as_f32(m);
+  const float s = amax_to_scale(amax, fp8_max<OUT>());
+  uint8_t* orow = out + row * (int64_t)row_vecs * kV;
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int j = tid + u * kBlock;
+    if (j < row_vecs) cast_vec<IN, OUT, false>(w[u], s, orow, j);
+  }
+  if (tid == 0) {
+    if (amax_out) amax_out[row] = amax;
+    if (scale_out) scale_out[row] = s;
+  }
+}
+
 // One workgroup per row; VEC selects 16-byte access (aligned rows) or element access.
 template <int IN, int OUT, bool VEC>
 __global__ __launch_bounds__(kBlock) void rowwise_block_kernel(const void* __restrict__ x, int64_t cols,
@@ -106,7 +151,19 @@ inline int launch_rowwise_impl(const void* x, int64_t rows, int64_t cols, void* 
   uint8_t* o = static_cast<uint8_t*>(out);
   const bool vec_ok = aligned(x, 16) && aligned(out, kStoreAlign) && cols % kV == 0;
   const int64_t row_vecs = cols / kV;
-  if (vec_ok && row_vecs <= 16 * kWave) {
+  const int64_t block_from = tuning("rowwise.block_from_vecs");  // rows at least this long take a workgroup each
+  if (vec_ok && row_vecs >= block_from && row_vecs <= 32 * kBlock && rows <= 0x7FFFFFFFll) {
+    const int rv = (int)row_vecs;
+#define DT_ROWB(NV) \
+  rowwise_block_resident_kernel<IN, OUT, NV><<<(unsigned)rows, kBlock, 0, stream>>>(x, rv, o, amax_out, scale_out)
+    if (row_vecs <= 1 * kBlock) DT_ROWB(1);
+    else if (row_vecs <= 2 * kBlock) DT_ROWB(2);
+    else if (row_vecs <= 4 * kBlock) DT_ROWB(4);
+    else if (row_vecs <= 8 * kBlock) DT_ROWB(8);
+    else if (row_vecs <= 16 * kBlock) DT_ROWB(16);
+    else DT_ROWB(32);
+#undef DT_ROWB
+  } else if (vec_ok && row_vecs <= 16 * kWave) {
     const unsigned grid = (unsigned)ceil_div(rows, kRowsPerBlock);
     const int rv = (int)row_vecs;
 #define DT_ROW(NV) rowwise_wave_kernel<IN, OUT, NV><<<grid, kBlock, 0, stream>>>(x, rows, rv, o, amax_out, scale_out)
