@@ -152,7 +152,7 @@ inline int launch_rowwise_impl(const void* x, int64_t rows, int64_t cols, void* 
   const bool vec_ok = aligned(x, 16) && aligned(out, kStoreAlign) && cols % kV == 0;
   const int64_t row_vecs = cols / kV;
   const int64_t block_from = tuning("rowwise.block_from_vecs");  // rows at least this long take a workgroup each
-  if (vec_ok && row_vecs >= block_from && row_vecs <= 32 * kBlock && rows <= 0x7FFFFFFFll) {
+  if (vec_ok && row_vecs >= block_from && row_vecs <= 64 * kBlock && rows <= 0x7FFFFFFFll) {
     const int rv = (int)row_vecs;
 #define DT_ROWB(NV) \
   rowwise_block_resident_kernel<IN, OUT, NV><<<(unsigned)rows, kBlock, 0, stream>>>(x, rv, o, amax_out, scale_out)
@@ -161,7 +161,8 @@ inline int launch_rowwise_impl(const void* x, int64_t rows, int64_t cols, void* 
     else if (row_vecs <= 4 * kBlock) DT_ROWB(4);
     else if (row_vecs <= 8 * kBlock) DT_ROWB(8);
     else if (row_vecs <= 16 * kBlock) DT_ROWB(16);
-    else DT_ROWB(32);
+    else if (row_vecs <= 32 * kBlock) DT_ROWB(32);
+    else DT_ROWB(64);
 #undef DT_ROWB
   } else if (vec_ok && row_vecs <= 16 * kWave) {
     const unsigned grid = (unsigned)ceil_div(rows, kRowsPerBlock);

@@ -299,9 +299,9 @@ def test_rowwise_shapes(d, in_dtype, fp8_dtype, shape):
 
 
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("vecs", [257, 300, 512, 513, 1024, 1030, 2048, 2500, 4096, 4100, 8192, 8193, 9000])
+@pytest.mark.parametrize("vecs", [257, 300, 512, 513, 1024, 1030, 2048, 2500, 4096, 4100, 8192, 8193, 9000, 16384, 16385])
 def test_rowwise_long_rows(d, in_dtype, vecs):
-    """rows of 257 ... 8192 sixteen-byte vectors get a workgroup each and stay in its registers (1 to 32
+    """rows of 257 ... 16384 sixteen-byte vectors get a workgroup each and stay in its registers (1 to 64
     vectors per lane, ragged last pass); longer ones are read twice.  Row maxima in the first and in the
     last vector of a row, an all-zero row, NaN in one row"""
     cols = vecs * (8 if in_dtype == torch.bfloat16 else 4)
