@@ -191,12 +191,12 @@ __device__ __forceinline__ void products_of(u32x4 w, float s, float (&p)[InTrait
   }
 }
 
+// one 16-byte vector of x -> kV / 4 words of fp8 bytes
 template <int IN, int OUT, bool ROUND_BF16, bool CHECK_NAN = true>
-__device__ __forceinline__ void cast_vec(u32x4 w, float s, uint8_t* __restrict__ out, int64_t vec_index) {
+__device__ __forceinline__ void cast_vec_to_words(u32x4 w, float s, uint32_t (&r)[InTraits<IN>::kVec / 4]) {
   constexpr int kV = InTraits<IN>::kVec;
   float p[kV];
   products_of<IN>(w, s, p);
-  uint32_t r[kV / 4];
   products_to_fp8<IN, OUT, ROUND_BF16>(p, r, 1.0f);
   if constexpr (CHECK_NAN) {  // rounding to bf16 keeps a NaN a NaN and its sign
     bool any_nan = false;
@@ -207,6 +207,12 @@ __device__ __forceinline__ void cast_vec(u32x4 w, float s, uint8_t* __restrict__
       for (int q = 0; q < kV / 4; ++q) r[q] = nan_patch4(r[q], p[4 * q], p[4 * q + 1], p[4 * q + 2], p[4 * q + 3]);
     }
   }
+}
+
+template <int IN, int OUT, bool ROUND_BF16, bool CHECK_NAN = true>
+__device__ __forceinline__ void cast_vec(u32x4 w, float s, uint8_t* __restrict__ out, int64_t vec_index) {
+  uint32_t r[InTraits<IN>::kVec / 4];
+  cast_vec_to_words<IN, OUT, ROUND_BF16, CHECK_NAN>(w, s, r);
   if constexpr (IN == DT_F32) st_stream(reinterpret_cast<uint32_t*>(out) + vec_index, r[0]);
   else st_stream(reinterpret_cast<u32x2*>(out) + vec_index, u32x2{r[0], r[1]});
 }
@@ -258,18 +264,45 @@ __global__ __launch_bounds__(kBlock) void cast_kernel(const void* __restrict__ x
   }
 }
 
-// Any alignment: one element per thread per step.
+// Any alignment (x aligned to its element, the outputs to a byte): the same 16-byte loads and packed
+// stores, through vector types that claim no more alignment than that.  The device serves such
+// accesses (unaligned access mode, the default for compute on ROCm); they cost the lines they
+// straddle.  8192^2 bf16 with x one element off: 182 us with one element per lane and step.
+typedef u32x4 u32x4_elem2 __attribute__((aligned(2)));
+typedef u32x4 u32x4_elem4 __attribute__((aligned(4)));
+typedef u32x2 u32x2_byte __attribute__((aligned(1)));
+typedef uint32_t u32_byte __attribute__((aligned(1)));
 template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR>
 __global__ __launch_bounds__(kBlock) void cast_kernel_unaligned(const void* __restrict__ x, int64_t numel,
                                                                 const float* __restrict__ scale,
                                                                 uint8_t* __restrict__ out, uint8_t* __restrict__ out2) {
+  constexpr int kV = InTraits<IN>::kVec;
   constexpr int OUT2 = OUT == DT_E4M3FN ? DT_E5M2 : DT_E4M3FN;
+  typedef typename std::conditional<IN == DT_F32, u32x4_elem4, u32x4_elem2>::type vec_t;
+  saturate_fp8_conversions();
   float s = scale[0], s2 = PAIR ? scale[1] : 0.f;
   if constexpr (ROUND_SCALE) { s = round_to_bf16(s); s2 = round_to_bf16(s2); }
+  const vec_t* v = static_cast<const vec_t*>(x);
+  const int64_t nvec = numel / kV, tail = numel % kV;
   const int64_t stride = (int64_t)gridDim.x * kBlock;
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < numel; i += stride) {
-    out[i] = cast_one<IN, OUT, ROUND_BF16>(x, i, s);
-    if constexpr (PAIR) out2[i] = cast_one<IN, OUT2, ROUND_BF16>(x, i, s2);
+  auto put = [](uint8_t* o, int64_t i, const uint32_t (&r)[kV / 4]) {
+    if constexpr (IN == DT_F32) *reinterpret_cast<u32_byte*>(o + i * 4) = r[0];
+    else *reinterpret_cast<u32x2_byte*>(o + i * 8) = u32x2{r[0], r[1]};
+  };
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += stride) {
+    const u32x4 w = v[i];
+    uint32_t r[kV / 4];
+    cast_vec_to_words<IN, OUT, ROUND_BF16>(w, s, r);
+    put(out, i, r);
+    if constexpr (PAIR) {
+      cast_vec_to_words<IN, OUT2, ROUND_BF16>(w, s2, r);
+      put(out2, i, r);
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < tail) {
+    const int64_t e = nvec * kV + threadIdx.x;
+    out[e] = cast_one<IN, OUT, ROUND_BF16>(x, e, s);
+    if constexpr (PAIR) out2[e] = cast_one<IN, OUT2, ROUND_BF16>(x, e, s2);
   }
 }
 
@@ -289,7 +322,7 @@ inline int launch_cast_impl(const void* x, int64_t numel, const float* scale, vo
     int grid = reduction_grid(nvec, kUnroll, PAIR ? "cast.pair_blocks_per_cu" : "cast.blocks_per_cu");
     cast_kernel<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR, kUnroll><<<grid, kBlock, 0, stream>>>(x, nvec, tail, scale, o, o2);
   } else {
-    int grid = reduction_grid(numel, 1, "cast.blocks_per_cu");
+    int grid = reduction_grid(numel / InTraits<IN>::kVec, 1, "cast.blocks_per_cu");
     cast_kernel_unaligned<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR><<<grid, kBlock, 0, stream>>>(x, numel, scale, o, o2);
   }
   return launch_status();
