@@ -57,22 +57,31 @@ __global__ __launch_bounds__(kBlock) void rowwise_wave_kernel(const void* __rest
 
 // Longer rows: one workgroup per row, NV vectors per lane kept in registers between the reduction
 // (one LDS exchange between the four waves) and the cast: still a single read of the row.
-template <int IN, int OUT, int NV>
+// ANY: rows that are not 16-byte aligned or not a whole number of vectors (cols % kV = tail elements,
+// done by the first lanes): the same loads and stores through vector types that claim only element /
+// byte alignment, as in cast_kernel_unaligned.
+template <int IN, int OUT, int NV, bool ANY = false>
 __global__ __launch_bounds__(kBlock) void rowwise_block_resident_kernel(const void* __restrict__ x, int row_vecs,
                                                                         uint8_t* __restrict__ out,
                                                                         float* __restrict__ amax_out,
-                                                                        float* __restrict__ scale_out) {
-  constexpr int kV = InTraits<IN>::kVec;
+                                                                        float* __restrict__ scale_out, int tail = 0) {
+  constexpr int kV = InTraits<IN>::kVec, kB = InTraits<IN>::kBytes;
   saturate_fp8_conversions();
   __shared__ uint32_t lds[kBlock / kWave];
   const int tid = threadIdx.x;
   const int64_t row = blockIdx.x;
-  const u32x4* v = static_cast<const u32x4*>(x) + row * row_vecs;
+  const int64_t cols = (int64_t)row_vecs * kV + tail;
+  const uint8_t* xrow = static_cast<const uint8_t*>(x) + row * cols * kB;
   u32x4 w[NV];
 #pragma unroll
   for (int u = 0; u < NV; ++u) {
     const int j = tid + u * kBlock;
-    w[u] = j < row_vecs ? ld_stream(v + j) : u32x4{0u, 0u, 0u, 0u};
+    if constexpr (ANY) {
+      typedef typename std::conditional<IN == DT_F32, u32x4_elem4, u32x4_elem2>::type vec_t;
+      w[u] = j < row_vecs ? reinterpret_cast<const vec_t*>(xrow)[j] : u32x4{0u, 0u, 0u, 0u};
+    } else {
+      w[u] = j < row_vecs ? ld_stream(reinterpret_cast<const u32x4*>(xrow) + j) : u32x4{0u, 0u, 0u, 0u};
+    }
   }
   uint32_t m = 0;
 #pragma unroll
@@ -85,14 +94,29 @@ __global__ __launch_bounds__(kBlock) void rowwise_block_resident_kernel(const vo
     }
   }
   if constexpr (IN != DT_F32) m = umax(m & 0xFFFFu, m >> 16) << 16;
+  if constexpr (ANY) {
+    if (tid < tail) m = umax(m, absbits_of<IN>(xrow, (int64_t)row_vecs * kV + tid));
+  }
   m = block_umax<kBlock / kWave>(m, lds);
   const float amax = as_f32(m);
   const float s = amax_to_scale(amax, fp8_max<OUT>());
-  uint8_t* orow = out + row * (int64_t)row_vecs * kV;
+  uint8_t* orow = out + row * cols;
 #pragma unroll
   for (int u = 0; u < NV; ++u) {
     const int j = tid + u * kBlock;
-    if (j < row_vecs) cast_vec<IN, OUT, false>(w[u], s, orow, j);
+    if (j < row_vecs) {
+      if constexpr (ANY) {
+        uint32_t r[kV / 4];
+        cast_vec_to_words<IN, OUT, false>(w[u], s, r);
+        if constexpr (IN == DT_F32) *reinterpret_cast<u32_byte*>(orow + (int64_t)j * 4) = r[0];
+        else *reinterpret_cast<u32x2_byte*>(orow + (int64_t)j * 8) = u32x2{r[0], r[1]};
+      } else {
+        cast_vec<IN, OUT, false>(w[u], s, orow, j);
+      }
+    }
+  }
+  if constexpr (ANY) {
+    if (tid < tail) orow[(int64_t)row_vecs * kV + tid] = cast_one<IN, OUT, false>(xrow, (int64_t)row_vecs * kV + tid, s);
   }
   if (tid == 0) {
     if (amax_out) amax_out[row] = amax;
@@ -164,6 +188,19 @@ inline int launch_rowwise_impl(const void* x, int64_t rows, int64_t cols, void* 
     else if (row_vecs <= 32 * kBlock) DT_ROWB(32);
     else DT_ROWB(64);
 #undef DT_ROWB
+  } else if (!vec_ok && row_vecs >= 1 && row_vecs <= 64 * kBlock && rows <= 0x7FFFFFFFll) {
+    // rows that are not aligned or not whole vectors: a workgroup per row with element-aligned vector accesses
+    const int rv = (int)row_vecs, tail = (int)(cols % kV);
+#define DT_ROWA(NV) \
+  rowwise_block_resident_kernel<IN, OUT, NV, true><<<(unsigned)rows, kBlock, 0, stream>>>(x, rv, o, amax_out, scale_out, tail)
+    if (row_vecs <= 1 * kBlock) DT_ROWA(1);
+    else if (row_vecs <= 2 * kBlock) DT_ROWA(2);
+    else if (row_vecs <= 4 * kBlock) DT_ROWA(4);
+    else if (row_vecs <= 8 * kBlock) DT_ROWA(8);
+    else if (row_vecs <= 16 * kBlock) DT_ROWA(16);
+    else if (row_vecs <= 32 * kBlock) DT_ROWA(32);
+    else DT_ROWA(64);
+#undef DT_ROWA
   } else if (vec_ok && row_vecs <= 16 * kWave) {
     const unsigned grid = (unsigned)ceil_div(rows, kRowsPerBlock);
     const int rv = (int)row_vecs;

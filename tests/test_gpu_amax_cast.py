@@ -299,23 +299,31 @@ def test_rowwise_shapes(d, in_dtype, fp8_dtype, shape):
 
 
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("vecs", [257, 300, 512, 513, 1024, 1030, 2048, 2500, 4096, 4100, 8192, 8193, 9000, 16384, 16385])
-def test_rowwise_long_rows(d, in_dtype, vecs):
+@pytest.mark.parametrize("extra", [0, 3])
+@pytest.mark.parametrize("vecs", [1, 40, 257, 300, 512, 513, 1024, 1030, 2048, 2500, 4096, 4100, 8192, 8193, 9000, 16384, 16385])
+def test_rowwise_long_rows(d, in_dtype, vecs, extra):
     """rows of 257 ... 16384 sixteen-byte vectors get a workgroup each and stay in its registers (1 to 64
     vectors per lane, ragged last pass); longer ones are read twice.  Row maxima in the first and in the
     last vector of a row, an all-zero row, NaN in one row"""
-    cols = vecs * (8 if in_dtype == torch.bfloat16 else 4)
+    # extra: a few elements past the last whole vector, which also leaves every row but the first misaligned
+    # (such rows take the same kernel with element-aligned vector accesses)
+    cols = vecs * (8 if in_dtype == torch.bfloat16 else 4) + extra
     a = util.rows_log_uniform_sigma((6, cols), 52 + vecs, in_dtype)
     a[1] = 0
     a[2, 0] = 3.0e4
     a[3, cols - 1] = -3.0e4
     a[4, cols // 2] = float("nan")
+    # the tensor itself one element off a 16-byte boundary as well
+    buf = torch.empty(a.numel() + 1, dtype=in_dtype, device="cuda")
+    buf[1:] = a.cuda().flatten()
+    shifted = buf[1:].view(a.shape)
     for fp8_dtype in FP8:
-        out, amax, scale = d.dynamic_scaled_quant_rowwise(a.cuda(), fp8_dtype)
         ref, ramax, rscale = co.dynamic_scaled_quant_rowwise(a, fp8_dtype)
-        assert torch.equal(amax.cpu().view(torch.int32), ramax.view(torch.int32))
-        assert torch.equal(scale.cpu().view(torch.int32), rscale.view(torch.int32))
-        assert torch.equal(util.codes(out), ref)
+        for src in (a.cuda(), shifted):
+            out, amax, scale = d.dynamic_scaled_quant_rowwise(src, fp8_dtype)
+            assert torch.equal(amax.cpu().view(torch.int32), ramax.view(torch.int32))
+            assert torch.equal(scale.cpu().view(torch.int32), rscale.view(torch.int32))
+            assert torch.equal(util.codes(out), ref)
 
 
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
