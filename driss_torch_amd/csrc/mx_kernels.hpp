@@ -148,7 +148,9 @@ __device__ __forceinline__ uint32_t vec_absmax_bits(u32x4 w) {
 // row -- because those are the scales that sit next to each other in the blocked layout: the 64
 // bytes of a pass then fall into 4 runs of 16 bytes instead of 16 runs of 4, which costs a
 // quarter of the memory transactions (36.8 -> 33 us at 8192 x 8192 bf16).
-template <int IN, int OUT, int LAYOUT, bool BAND4 = false>
+// XANY: x is only aligned to its element (a view that starts at an odd element): the same 16-byte
+// loads through a vector type that claims no more (the device serves them).
+template <int IN, int OUT, int LAYOUT, bool BAND4 = false, bool XANY = false>
 __global__ __launch_bounds__(kBlock) void mx_row_kernel(const void* __restrict__ x, uint32_t nblocks,
                                                         uint32_t kblocks, uint8_t* __restrict__ data,
                                                         uint8_t* __restrict__ scale) {
@@ -182,7 +184,12 @@ __global__ __launch_bounds__(kBlock) void mx_row_kernel(const void* __restrict__
 #pragma unroll
     for (int c = 0; c < LPB; ++c) {
       const uint32_t vi = vec_index(c);
-      w[c] = vi < nvec ? ld_stream(v + vi) : u32x4{0u, 0u, 0u, 0u};
+      if constexpr (XANY) {
+        typedef typename std::conditional<IN == DT_F32, u32x4_elem4, u32x4_elem2>::type vec_t;
+        w[c] = vi < nvec ? reinterpret_cast<const vec_t*>(x)[vi] : u32x4{0u, 0u, 0u, 0u};
+      } else {
+        w[c] = vi < nvec ? ld_stream(v + vi) : u32x4{0u, 0u, 0u, 0u};
+      }
     }
     uint32_t mybyte = 0;
 #pragma unroll

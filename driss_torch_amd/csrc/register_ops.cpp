@@ -239,7 +239,6 @@ std::tuple<Tensor, Tensor> mx_fp8_quantize_ex(const Tensor& input, int64_t block
   const int64_t scale_elems = blocked ? dt_blocked_scale_bytes(other_dim, blocked_dim / 32) : total_blocks;
   Tensor scale = at::empty({scale_elems}, input.options().dtype(at::kFloat8_e8m0fnu));
   if (input.numel() == 0) return {data, scale};
-  TORCH_CHECK(reinterpret_cast<std::uintptr_t>(input.data_ptr()) % 16 == 0, "Input tensor must be 16-byte aligned");
   check_status(dt_mx_fp8_quantize(input.data_ptr(), in_code(input), m, n, ax, transpose ? 1 : 0, out_code(fp8_type),
                                   blocked ? DT_SCALE_BLOCKED : DT_SCALE_PLAIN, data.data_ptr(),
                                   static_cast<uint8_t*>(scale.data_ptr()), ctx.stream),
@@ -268,7 +267,6 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> mx_fp8_quantize_dual(const Tensor& in
   Tensor scale_r = at::empty({blocked ? dt_blocked_scale_bytes(m, n / 32) : m * (n / 32)}, e8);
   Tensor scale_c = at::empty({blocked ? dt_blocked_scale_bytes(n, m / 32) : n * (m / 32)}, e8);
   if (input.numel() == 0) return {data_r, scale_r, data_c, scale_c};
-  TORCH_CHECK(reinterpret_cast<std::uintptr_t>(input.data_ptr()) % 16 == 0, "Input tensor must be 16-byte aligned");
   check_status(dt_mx_fp8_quantize_dual(input.data_ptr(), in_code(input), m, n, out_code(fp8_type),
                                        blocked ? DT_SCALE_BLOCKED : DT_SCALE_PLAIN, data_r.data_ptr(),
                                        static_cast<uint8_t*>(scale_r.data_ptr()), data_c.data_ptr(),

@@ -77,6 +77,30 @@ def test_mx_cast_special_blocks(d, in_dtype, axis, transpose):
     assert torch.equal(util.codes(data), rd)
 
 
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_mx_cast_input_off_a_16_byte_boundary(d, in_dtype):
+    """a contiguous view that starts one element into its buffer: the row-wise cast keeps its 16-byte
+    loads (element-aligned vector type), the other orientations go through the generic kernel; all
+    of them against the oracle"""
+    rows, cols = 96, 544
+    a = util.student_t((rows, cols), 61, in_dtype)
+    buf = torch.empty(a.numel() + 3, dtype=in_dtype, device="cuda")
+    buf[1:1 + a.numel()] = a.cuda().flatten()
+    x = buf[1:1 + a.numel()].view(rows, cols)
+    assert x.data_ptr() % 16 != 0
+    rd, rs = co.mx_quantize(a, 1, False)
+    data, scale = d.mx_fp8_quantize(x)
+    assert torch.equal(util.codes(data), rd) and torch.equal(util.codes(scale), rs.flatten())
+    data, scale = d.mx_fp8_quantize_blocked(x)
+    assert torch.equal(util.codes(data), rd) and torch.equal(util.codes(scale), co.to_blocked(rs))
+    cd, cs = co.mx_quantize(a, 0, True)
+    data, scale = d.mx_fp8_quantize(x, 32, 0, True)
+    assert torch.equal(util.codes(data), cd) and torch.equal(util.codes(scale), cs.flatten())
+    dr, sr, dc, sc = d.mx_fp8_quantize_dual(x)   # falls back to the two single casts
+    assert torch.equal(util.codes(dr), rd) and torch.equal(util.codes(sr), rs.flatten())
+    assert torch.equal(util.codes(dc), cd) and torch.equal(util.codes(sc), cs.flatten())
+
+
 def test_mx_cast_blocked_scales_and_errors(d, cabi):
     for shape, axis in [((256, 512), 1), ((129, 160), 1), ((512, 256), 0), ((160, 129 * 1), 0), ((96, 200), 0)]:
         a = util.student_t(shape, 71 + shape[0])
