@@ -143,7 +143,10 @@ DT_API int dt_dynamic_scaled_quant_rowwise(const void* x, int in_dtype, int64_t 
  * scale_layout DT_SCALE_BLOCKED writes the scale matrix directly in the layout
  * dt_mx_fp8_bf16 reads (dt_blocked_scale_bytes(scale_rows, scale_cols) bytes, padding
  * zeroed); it needs the scale matrix to be [outer, inner/32], i.e. (axis 1, transpose 0)
- * or (axis 0, transpose 1).  x must be 16-byte aligned; in_dtype F32, BF16 or F16.        */
+ * or (axis 0, transpose 1).  in_dtype F32, BF16 or F16.  x aligned to its element: the fast
+ * kernels want 16 bytes; an x off a 16-byte boundary keeps its vector loads for (axis 1,
+ * transpose 0) and takes a much slower general kernel for the other orientations, as does
+ * (axis 1, transpose 1) always.                                                            */
 DT_API int dt_mx_fp8_quantize(const void* x, int in_dtype, int64_t rows, int64_t cols, int axis,
                               int transpose, int out_dtype, int scale_layout, void* data,
                               uint8_t* scale, dt_stream_t stream);
