@@ -29,11 +29,30 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 FP8_PEAK_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 FP4_PEAK_TFLOPS = 10100.0   # MI355X dense fp4 MFMA
 MALL_BYTES = 256 << 20
-# HBM-side bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, each
-# scaled by what the same counter reads for a plain 128 MiB device copy (fetch x1.9996, write
-# x1.0): profiles/dynamic_quant_pair_config2_hbm_traffic.txt
-CAST_PAIR_TRAFFIC_BYTES = 268.57e6
-RESIDENT_PAIR_TRAFFIC_BYTES = 269.38e6  # same method, resident_quant_kernel (one read of x, two fp8 writes)
+# HBM-side bytes per launch of the step's kernels, from rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled
+# by what the same counter reads for a plain 128 MiB device copy: the summary of those two counter
+# runs is a text file, read at run time (its commands are in its header)
+TRAFFIC_PROFILE = ROOT / "profiles" / "dynamic_quant_pair_config2_hbm_traffic.txt"
+
+
+def traffic_from_profile(kernel_prefix):
+    """HBM bytes per launch of the kernel whose name starts with `kernel_prefix`, or None."""
+    try:
+        for line in TRAFFIC_PROFILE.read_text().splitlines():
+            if line.startswith(kernel_prefix):
+                return float(line.split()[-1]) * 1e6  # last column: traffic in MB
+    except (OSError, ValueError):
+        pass
+    return None
+
+
+def normal_with_outliers(torch, shape, seed, frac=1e-3, factor=100.0):
+    """config 2's input: N(0,1) drawn in fp32 on the CPU, 0.1 % of the positions multiplied by 100, as bf16"""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(shape, generator=g)
+    idx = torch.randperm(x.numel(), generator=g)[:max(1, round(frac * x.numel()))]
+    x.view(-1)[idx] *= factor
+    return x.to(torch.bfloat16)
 
 
 def _events(n):
@@ -72,6 +91,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--gemm-only", action="store_true",
                     help="run only the block-scaled GEMM rows of the per-kernel table (for profiling) and print them")
+    ap.add_argument("--phases", action="store_true",
+                    help="also report the per-phase times of the step's kernel (shader clock counter readings it dumps)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain device copies of 128 MiB (to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
@@ -83,24 +104,28 @@ def main():
     import torch
 
     from driss_torch_amd import cabi
-    from tests import util
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     K, W = args.steps, args.warmup
     if args.gemm_only:
-        print(json.dumps({"kernels": extra_kernels(torch, cabi, util, dev, K, W, gemm_only=True)}))
+        print(json.dumps({"kernels": extra_kernels(torch, cabi, dev, K, W, gemm_only=True)}))
         return
 
     # ------------------------------------------------------------ headline step: config 2
     R = C = 8192
     numel = R * C
-    step_bytes = numel * (2 + 2 + 1 + 1)          # two reads of x, two fp8 writes
-    cast_bytes = numel * (2 + 1 + 1)              # dominant kernel: one read, two writes
-    amax_bytes = numel * 2
+    # Bytes of the step.  The survey's per-unit figure for the path counts x twice (one read for the
+    # reduction, one for the cast: 6 B per element with two fp8 outputs); the step's one kernel keeps
+    # x on the chip between its passes, so what it must move -- and what the counters see -- is one
+    # read of x and the two fp8 outputs: 4 B per element.  `value` and the roofline are quoted on
+    # those 4 B; the 6 B figure is reported beside them as the two-pass equivalent.
+    two_pass_bytes = numel * (2 + 2 + 1 + 1)
+    step_bytes = numel * (2 + 1 + 1)
+    cast_bytes = numel * (2 + 1 + 1)              # the cast of the two-kernel path: one read, two writes
     ns = nsets_for(numel * 4)
-    x_cpu = util.normal_with_outliers((R, C), 1002)
+    x_cpu = normal_with_outliers(torch, (R, C), 1002)
     xs = [x_cpu.to(dev) if i == 0 else torch.roll(x_cpu, i, 0).to(dev) for i in range(ns)]
     o4 = [torch.empty((R, C), dtype=torch.float8_e4m3fn, device=dev) for _ in range(ns)]
     o5 = [torch.empty((R, C), dtype=torch.float8_e5m2, device=dev) for _ in range(ns)]
@@ -137,6 +162,8 @@ def main():
     step_us = time_launches(step, ns, K, 0)
     step_gbs = step_bytes / (step_us * 1e-6) / 1e9
 
+    phases = resident_phases(torch, cabi, step, ns) if args.phases else None
+
     # for comparison: the two-kernel path every larger tensor takes (amax, then cast), the cast
     # bracketed by an event pair per launch (adds about 4 us of dispatch latency to it)
     cabi.set_tuning("dynamic.resident", 0)
@@ -149,6 +176,8 @@ def main():
     cast_us = statistics.fmean(e[0].elapsed_time(e[1]) for e in evs) * 1e3
     cabi.set_tuning("dynamic.resident", 1)
 
+    traffic = traffic_from_profile("dt::resident_quant_kernel")
+    cast_traffic = traffic_from_profile("dt::cast_kernel")
     result = {
         "metric": "cast/amax HBM GB/s (% of 8 TB/s) at 8192² bf16; MXFP8 GEMM TFLOPS",
         "value": round(value, 1),
@@ -163,23 +192,30 @@ def main():
         "dtype": "bf16->fp8 (fp32 arithmetic)",
         "data": "synthetic",
         "config": {"workload": "config 2: amax + dynamic_scaled_quant per tensor, bf16 [8192,8192] N(0,1) with 0.1% x100 "
-                               "outliers -> fp32 amax, scales, e4m3fn and e5m2 (402.7 MB algorithmic per step)",
+                               "outliers -> fp32 amax, scales, e4m3fn and e5m2; value counts the 268.4 MB the step must "
+                               "move (x once, two fp8 outputs)",
                    "buffer_sets": ns, "product_rounding": "bf16 product, bf16-rounded scale (eager with a 0-dim scale)"},
-        # achieved = algorithmic bytes of the step (x read for the reduction, x read for the cast, two
-        # fp8 outputs: 6 B per element) / kernel time.  The kernel keeps x in registers and LDS between
-        # the two passes, so HBM sees x once: `traffic` (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a
-        # plain copy) is 4 B per element, and frac can exceed 1.
+        # achieved = the bytes the kernel must move (x once + two fp8 outputs: 4 B per element, its lower
+        # bound) / average launch time, so frac is a fraction of the HBM peak and cannot exceed 1.  `traffic`
+        # is what rocprofv3 FETCH_SIZE + WRITE_SIZE saw per launch (scaled by a plain copy), read from the
+        # committed summary of those runs.  The survey's 6 B per element (x read by the reduction and again
+        # by the cast, as two kernels would) over the same time is two_pass_equivalent_GBs.
         "roofline": {"kernel": "resident_quant_kernel<bf16, e4m3fn+e5m2 pair>", "bound": "hbm", "achieved": round(step_gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(step_gbs / HBM_PEAK_GBS, 4),
                      "avg_launch_us": round(step_us, 2), "algorithmic_bytes_per_launch": step_bytes,
-                     "traffic": RESIDENT_PAIR_TRAFFIC_BYTES,
-                     "traffic_rate_GBs": round(RESIDENT_PAIR_TRAFFIC_BYTES / (step_us * 1e-6) / 1e9, 1)},
+                     "min_traffic_bytes": step_bytes, "frac_of_min_traffic": round(step_gbs / HBM_PEAK_GBS, 4),
+                     "traffic": traffic, "traffic_source": str(TRAFFIC_PROFILE.relative_to(ROOT)) if traffic else None,
+                     "traffic_rate_GBs": round(traffic / (step_us * 1e-6) / 1e9, 1) if traffic else None,
+                     "two_pass_algorithmic_bytes": two_pass_bytes,
+                     "two_pass_equivalent_GBs": round(two_pass_bytes / (step_us * 1e-6) / 1e9, 1)},
         "two_kernel_path": {"step_us": round(two_kernel_us, 2),
-                            "GBs": round(step_bytes / (two_kernel_us * 1e-6) / 1e9, 1),
+                            "GBs of the 6 B per element its two kernels read and write": round(two_pass_bytes / (two_kernel_us * 1e-6) / 1e9, 1),
                             "cast_kernel(pair) inside the step, event pair per launch, us": round(cast_us, 2),
                             "cast_kernel(pair) GBs (4 B per element)": round(cast_bytes / (cast_us * 1e-6) / 1e9, 1),
-                            "cast_kernel(pair) traffic": CAST_PAIR_TRAFFIC_BYTES},
+                            "cast_kernel(pair) traffic": cast_traffic},
     }
+    if phases:
+        result["resident_phases"] = phases
     if args.calibrate_copy:
         src = xs[0]
         dst = torch.empty_like(src)
@@ -191,13 +227,58 @@ def main():
     torch.cuda.empty_cache()
 
     if not args.no_extra:
-        result["kernels"] = extra_kernels(torch, cabi, util, dev, K, W)
+        result["kernels"] = extra_kernels(torch, cabi, dev, K, W)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, x_cpu, step_bytes)
     print(json.dumps(result))
 
 
-def extra_kernels(torch, cabi, util, dev, K, W, gemm_only=False):
+def resident_phases(torch, cabi, step, ns, launches=20):
+    """Where the step's one kernel spends its time: every workgroup writes four readings of the 100 MHz
+    constant-rate counter (start, share loaded and reduced, released from the grid barrier, stores
+    done; dt_set_phase_log), collected here over `launches` launches with a synchronisation after each.
+    All figures in microseconds, medians over the launches; t = 0 is the first workgroup's start."""
+    L = cabi.lib()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    log = torch.zeros((cus, 4), dtype=torch.int64, device="cuda")
+    assert L.dt_set_phase_log(log.data_ptr(), log.numel() * 8) == 0
+    rows = []
+    try:
+        for i in range(launches + 3):
+            log.zero_()
+            step(i % ns)
+            torch.cuda.synchronize()
+            t = log.cpu().double()
+            t = t[t[:, 0] > 0]  # workgroups of the grid
+            if i < 3 or t.numel() == 0:
+                continue
+            t = (t - t[:, 0].min()) / 100.0  # 100 MHz -> us
+            med = lambda v: float(v.median())  # noqa: E731
+            rows.append({
+                "workgroups": int(t.shape[0]),
+                "last_workgroup_starts_at": float(t[:, 0].max()),
+                "load_and_reduce_per_workgroup_median": med(t[:, 1] - t[:, 0]),
+                "first_workgroup_loaded_at": float(t[:, 1].min()),
+                "last_workgroup_loaded_at": float(t[:, 1].max()),
+                "released_at_median": med(t[:, 2]),
+                "released_at_last": float(t[:, 2].max()),
+                "wait_in_barrier_per_workgroup_median": med(t[:, 2] - t[:, 1]),
+                "release_after_last_arrival_median": med(t[:, 2]) - float(t[:, 1].max()),
+                "convert_and_store_per_workgroup_median": med(t[:, 3] - t[:, 2]),
+                "first_workgroup_done_at": float(t[:, 3].min()),
+                "last_workgroup_done_at": float(t[:, 3].max()),
+            })
+    finally:
+        L.dt_set_phase_log(None, 0)
+    if not rows:
+        return None
+    out = {k: round(statistics.median(r[k] for r in rows), 2) for k in rows[0]}
+    out["launches"] = len(rows)
+    out["unit"] = "us (100 MHz counter, 0.01 us resolution)"
+    return out
+
+
+def extra_kernels(torch, cabi, dev, K, W, gemm_only=False):
     """Every other kernel of the path at its benchmark config: rotated (HBM) and hot-cache."""
     rows = []
 

@@ -18,7 +18,6 @@ for _p in (hip_lib_path, lib_path):
     if not _p.exists():
         raise ImportError(f"{_p} is missing: build it with `python driss_torch_amd/_build.py`")
 torch.ops.load_library(str(lib_path.resolve()))
-torch.ops.import_module("driss_torch_amd.abstract_impls")
 
 ops = torch.ops.DrissTorch
 Tensor = torch.Tensor
@@ -138,3 +137,8 @@ def mx_fp4_quantize(input: Tensor, blocked: bool = False, axis: int = 1) -> Tupl
 def to_blocked(scale: Tensor) -> Tensor:
     """[R, C] E8M0 scale matrix -> flat blocked 128x4 layout (zero padded)."""
     return ops.to_blocked(scale)
+
+
+# The fake implementations register from the module the operator library names as their home
+# (the reference's: src/register_ops.cpp:14).  Imported last: that package re-exports the wrappers above.
+torch.ops.import_module("driss_torch.abstract_impls")

@@ -52,8 +52,11 @@ def time_us(fn, *args, min_run_s: float = 0.05) -> float:
         n *= 4
 
 
-def run(compiled: bool):
-    from driss_torch_amd import saturated_cast
+def run(compiled: bool, timed: bool = True, on_checked=None):
+    """One row per (shape, fp8 dtype): the correctness check of the reference's harness
+    (benchmarks/benchmark_saturated_casting.py:100-108), then, if `timed`, the timings (:110-128).
+    `on_checked(x, scale, fp8_dtype, out)` is called after each check (a test hooks in there)."""
+    from driss_torch import saturated_cast  # the reference's import (benchmarks/benchmark_saturated_casting.py:8)
 
     rows = []
     for (r, c), lp in itertools.product(SHAPES, LOW_PRECISION):
@@ -62,15 +65,19 @@ def run(compiled: bool):
         out = saturated_cast(x, scale, lp)
         ref = eager_scaled_quant(x, scale, lp)
         torch.testing.assert_close(out.to(torch.bfloat16), ref.to(torch.bfloat16), rtol=1e-3, atol=1e-3)
-        hip_us = time_us(saturated_cast, x, scale, lp)
-        eager_us = time_us(eager_scaled_quant, x, scale, lp)
-        row = {"num_rows": r, "num_cols": c, "high_precision_dtype": "bfloat16", "low_precision_dtype": str(lp).split(".")[-1],
-               "hip_time_us": round(hip_us, 2), "pytorch_time_us": round(eager_us, 2),
-               "hip_GBps": round(r * c * 3 / hip_us / 1e3, 1), "speedup_vs_eager": round(eager_us / hip_us, 2)}
-        if compiled:
-            fn = torch.compile(eager_scaled_quant, fullgraph=True)
-            row["compiled_pytorch_time_us"] = round(time_us(fn, x, scale, lp), 2)
+        if on_checked is not None:
+            on_checked(x, scale, lp, out)
+        row = {"num_rows": r, "num_cols": c, "high_precision_dtype": "bfloat16", "low_precision_dtype": str(lp).split(".")[-1]}
+        if timed:
+            hip_us = time_us(saturated_cast, x, scale, lp)
+            eager_us = time_us(eager_scaled_quant, x, scale, lp)
+            row.update({"hip_time_us": round(hip_us, 2), "pytorch_time_us": round(eager_us, 2),
+                        "hip_GBps": round(r * c * 3 / hip_us / 1e3, 1), "speedup_vs_eager": round(eager_us / hip_us, 2)})
+            if compiled:
+                fn = torch.compile(eager_scaled_quant, fullgraph=True)
+                row["compiled_pytorch_time_us"] = round(time_us(fn, x, scale, lp), 2)
         rows.append(row)
+        del x, out, ref
     return rows
 
 

@@ -47,6 +47,8 @@ SIGNATURES = {
     "dt_mx_gemm_workspace_init": (_i32, [_vp, _sz, _vp]),
     "dt_mx_fp8_bf16_ws": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "dt_mx_fp4_bf16_ws": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "dt_dynamic_quant_gave_up": (_i32, []),
+    "dt_set_phase_log": (_i32, [_vp, _sz]),
     "dt_set_tuning": (_i32, [_cp, _i32]),
     "dt_get_tuning": (_i32, [_cp, C.POINTER(_i32)]),
 }

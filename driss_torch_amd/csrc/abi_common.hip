@@ -98,6 +98,9 @@ const char* dt_status_string(int status) {
     case DT_ERR_INVALID_MODE: return "invalid mode";
     case DT_ERR_LAUNCH: return "kernel launch failed";
     case DT_ERR_EMPTY: return "reduction over zero elements";
+    case DT_ERR_RESIDENT_GAVE_UP:
+      return "an earlier dynamic quantization on this device gave up waiting for the whole chip and wrote NaN "
+             "(is another process using the GPU?); the one-kernel path is now off for this process";
     default: return "unknown status";
   }
 }

@@ -21,9 +21,9 @@ extern "C" int dt_dynamic_scaled_quant(const void* x, int in_dtype, int64_t nume
   if (int st = dt::check_workspace(workspace, workspace_bytes)) return st;
   hipStream_t s = dt::as_hip(stream);
   const float fm = fmax_of(out_dtype);
-  if (dt::launch_resident<false>(x, in_dtype, numel, out_dtype, round_mode, workspace, out, nullptr, amax_out, scale_out, fm,
-                                 0.f, s) == DT_OK)
-    return DT_OK;
+  const int res = dt::launch_resident<false>(x, in_dtype, numel, out_dtype, round_mode, workspace, out, nullptr, amax_out,
+                                             scale_out, fm, 0.f, s);
+  if (res == DT_OK || res == DT_ERR_RESIDENT_GAVE_UP) return res;
   int st = in_dtype == DT_F32 ? dt::launch_amax<DT_F32>(x, numel, workspace, amax_out, scale_out, 1, fm, 0.f, s)
                               : dt::launch_amax<DT_BF16>(x, numel, workspace, amax_out, scale_out, 1, fm, 0.f, s);
   if (st) return st;
@@ -59,10 +59,11 @@ extern "C" int dt_dynamic_scaled_quant_pair(const void* x, int in_dtype, int64_t
                                             void* workspace, size_t workspace_bytes, dt_stream_t stream) {
   if (int st = dt::check_cast_args(x, in_dtype, numel, DT_E4M3FN, round_mode, out_e4m3fn)) return st;
   if (!out_e5m2) return DT_ERR_NULL_POINTER;
-  if (numel > 0 && dt::check_workspace(workspace, workspace_bytes) == DT_OK && (in_dtype == DT_F32 || in_dtype == DT_BF16) &&
-      dt::launch_resident<true>(x, in_dtype, numel, DT_E4M3FN, round_mode, workspace, out_e4m3fn, out_e5m2, amax_out,
-                                scale_out, 448.0f, 57344.0f, dt::as_hip(stream)) == DT_OK)
-    return DT_OK;
+  if (numel > 0 && dt::check_workspace(workspace, workspace_bytes) == DT_OK && (in_dtype == DT_F32 || in_dtype == DT_BF16)) {
+    const int res = dt::launch_resident<true>(x, in_dtype, numel, DT_E4M3FN, round_mode, workspace, out_e4m3fn, out_e5m2,
+                                              amax_out, scale_out, 448.0f, 57344.0f, dt::as_hip(stream));
+    if (res == DT_OK || res == DT_ERR_RESIDENT_GAVE_UP) return res;
+  }
   if (int st = dt_amax_scales(x, in_dtype, numel, amax_out, scale_out, workspace, workspace_bytes, stream)) return st;
   const float* scale = reinterpret_cast<const float*>(static_cast<const uint8_t*>(workspace) + dt::kWsScale);
   return dt::launch_cast<true>(x, in_dtype, numel, scale, DT_E4M3FN, round_mode, out_e4m3fn, out_e5m2, dt::as_hip(stream));
@@ -78,4 +79,14 @@ extern "C" int dt_dynamic_scaled_quant_rowwise(const void* x, int in_dtype, int6
   if (!x || !out) return DT_ERR_NULL_POINTER;
   if (!dt::aligned(x, in_dtype == DT_F32 ? 4 : 2)) return DT_ERR_MISALIGNED;
   return dt::launch_rowwise(x, in_dtype, rows, cols, out_dtype, out, amax_out, scale_out, dt::as_hip(stream));
+}
+
+extern "C" int dt_dynamic_quant_gave_up(void) { return dt::resident_take_gave_up() ? 1 : 0; }
+
+extern "C" int dt_set_phase_log(void* device_buffer, size_t bytes) {
+  if (device_buffer && !dt::aligned(device_buffer, 8)) return DT_ERR_MISALIGNED;
+  dt::ResidentGate& gate = dt::resident_gate();
+  gate.phase_log_bytes.store(device_buffer ? bytes : 0, std::memory_order_relaxed);
+  gate.phase_log.store(static_cast<uint64_t*>(device_buffer), std::memory_order_relaxed);
+  return DT_OK;
 }

@@ -418,7 +418,7 @@ Tensor sweep_mm(Tensor, Tensor, Tensor, Tensor, std::optional<Tensor>, at::Scala
 }  // namespace driss_torch
 
 TORCH_LIBRARY(DrissTorch, m) {
-  m.impl_abstract_pystub("driss_torch_amd.abstract_impls");
+  m.impl_abstract_pystub("driss_torch.abstract_impls");  // src/register_ops.cpp:14
   m.def("keyed_random_uniform(Tensor keys, int cols) -> Tensor");
   m.impl("keyed_random_uniform", c10::DispatchKey::CUDA, TORCH_FN(driss_torch::keyed_random_uniform));
   m.def("saturated_cast(Tensor input, Tensor scale, ScalarType dtype, bool transpose) -> Tensor");

@@ -19,8 +19,9 @@
 // end of the kernel whatever happens.
 #pragma once
 
-#include <atomic>
+#include <stdlib.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "quant_kernels.hpp"
@@ -67,7 +68,8 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
                                                                uint8_t* __restrict__ ws, uint8_t* __restrict__ out,
                                                                uint8_t* __restrict__ out2, float* __restrict__ amax_out,
                                                                float* __restrict__ scale_out, float fmax0, float fmax1,
-                                                               uint32_t spin_limit) {
+                                                               uint32_t spin_limit, uint32_t* __restrict__ host_flag,
+                                                               uint64_t* __restrict__ phase_log) {
   constexpr int kV = InTraits<IN>::kVec;
   constexpr int OUT2 = OUT == DT_E4M3FN ? DT_E5M2 : DT_E4M3FN;
   extern __shared__ __attribute__((aligned(16))) u32x4 keep[];  // [kResLdsVecs][kBlock]
@@ -78,6 +80,13 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
   const u32x4* v = static_cast<const u32x4*>(x);
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   const int64_t first = (int64_t)blockIdx.x * kBlock + tid;
+  // phase_log (normally null): four readings of the constant-rate 100 MHz counter per workgroup --
+  // start, share loaded and reduced, released from the grid barrier, done -- for the benchmark's
+  // per-phase report.  The counter is common to all CUs, so readings of different workgroups compare.
+  auto stamp = [&](int k) {
+    if (phase_log && tid == 0) phase_log[blockIdx.x * 4 + k] = wall_clock64();
+  };
+  stamp(0);
 
   // ---- pass 1: load the share once, keep it, reduce |x|
   u32x4 r[kResRegVecs];
@@ -155,6 +164,7 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
   }
   if (blockIdx.x == 0 && tid < tail) m = umax(m, absbits_of<IN>(x, nvec * kV + tid));  // x is 16-byte aligned: no head
   m = block_umax<kBlock / kWave>(m, red);
+  stamp(1);
 
   // ---- grid barrier on the reduction's atomics: fold the partial into the running maximum,
   // take a ticket, wait until every workgroup has taken one, read the maximum.  The last
@@ -170,11 +180,14 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
     uint32_t one = 1u;  // the ticket depends on the returned value, so the two atomics stay ordered
     asm volatile("v_and_or_b32 %0, %1, 0, %0" : "+v"(one) : "v"(before));
     const uint32_t t = __hip_atomic_fetch_add(ticket, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    uint32_t bits;
+    uint32_t bits, released = 0u;
     if (t == gridDim.x - 1) {
       // last to arrive: every other workgroup's maximum was folded in before it took its ticket
       bits = __hip_atomic_load(running, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(release, (1ull << 32) | bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // an exchange, not a store: its returned value (always 0) is folded into the departure below, so
+      // this workgroup cannot be counted as departed -- and the release word cannot be re-armed by the
+      // last one to leave -- before the release has been performed
+      released = (uint32_t)__hip_atomic_exchange(release, (1ull << 32) | bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else {
       uint32_t spins = 0;
       uint64_t rel;
@@ -182,6 +195,8 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
         __builtin_amdgcn_s_sleep(2);
         if (++spins >= spin_limit) {  // cannot happen when the grid is resident; never hang the GPU
           __hip_atomic_store(reinterpret_cast<uint32_t*>(ws + kWsTimeout), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          // and tell the host (a word of pinned host memory): the library's next call on this device reports it
+          if (host_flag) __hip_atomic_store(host_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
           rel = 0x7FC00000ull;  // the outputs of this workgroup become NaN: a loud failure
           break;
         }
@@ -191,6 +206,7 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
     bcast = bits;
     uint32_t dep = 1u;
     asm volatile("v_and_or_b32 %0, %1, 0, %0" : "+v"(dep) : "v"(bits));  // leave only after the read
+    asm volatile("v_and_or_b32 %0, %1, 0, %0" : "+v"(dep) : "v"(released));  // ... and after the release
     if (__hip_atomic_fetch_add(depart, dep, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1) {
       __hip_atomic_store(running, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(depart, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -211,6 +227,7 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
     }
   }
   __syncthreads();
+  stamp(2);
   const float amax = as_f32(bcast);
   float s = amax_to_scale(amax, fmax0), s2 = PAIR ? amax_to_scale(amax, fmax1) : 0.f;
   if constexpr (ROUND_SCALE) { s = round_to_bf16(s); s2 = round_to_bf16(s2); }
@@ -277,6 +294,11 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
     out[e] = cast_one<IN, OUT, ROUND_BF16>(x, e, s);
     if constexpr (PAIR) out2[e] = cast_one<IN, OUT2, ROUND_BF16>(x, e, s2);
   }
+  if (phase_log) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores of this wave have left
+    __syncthreads();
+    stamp(3);
+  }
 }
 
 // Host-side chaining of resident launches (see launch_resident_impl).
@@ -286,10 +308,45 @@ struct ResidentGate {
   bool used[kMaxDevices] = {};
   hipStream_t last_stream[kMaxDevices] = {};  // stream of the device's latest resident launch
   hipEvent_t event[kMaxDevices] = {};         // recorded there when a launch arrives on another stream
+  // One word of pinned host memory per device, made at the device's first resident launch and kept for
+  // the life of the process: a workgroup that gives up waiting sets it, the host reads it before the
+  // next per-tensor dynamic quantization on that device.
+  volatile uint32_t* gave_up_host[kMaxDevices] = {};
+  uint32_t* gave_up_dev[kMaxDevices] = {};
+  // device buffer for the per-phase clock readings of the next resident launches (benchmarking), or null
+  std::atomic<uint64_t*> phase_log{nullptr};
+  std::atomic<size_t> phase_log_bytes{0};
 };
 inline ResidentGate& resident_gate() {
   static ResidentGate* g = new ResidentGate();  // leaked on purpose: no HIP calls at process exit
   return *g;
+}
+
+// True when the process runs under a CU mask given through the environment, which
+// hipExtStreamGetCUMask does not report: the grid might then never be resident as a whole.
+inline bool cu_mask_in_environment() {
+  static const bool masked = [] {
+    for (const char* name : {"HSA_CU_MASK", "ROC_GLOBAL_CU_MASK", "HSA_CU_MASK_SKIP_INIT"}) {
+      const char* v = getenv(name);
+      if (v && *v) return true;
+    }
+    return false;
+  }();
+  return masked;
+}
+
+// Has a resident launch on the current device given up since the last time this was asked?  Reads and
+// clears the host word; meaningful once the launch in question has completed.
+inline bool resident_take_gave_up() {
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  if (dev < 0 || dev >= ResidentGate::kMaxDevices) return false;
+  ResidentGate& gate = resident_gate();
+  std::lock_guard<std::mutex> lock(gate.mu);
+  volatile uint32_t* w = gate.gave_up_host[dev];
+  if (!w || *w == 0u) return false;
+  *w = 0u;
+  return true;
 }
 
 // CUs a stream may use: all of them, unless it was created with a CU mask
@@ -360,7 +417,20 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
   }
   // every workgroup waits for all the others: a stream that may not use as many CUs as the grid has
   // workgroups could never hold them all at once
-  if (stream_cu_count(stream) < grid) return kResidentNotTaken;
+  if (stream_cu_count(stream) < grid || cu_mask_in_environment()) return kResidentNotTaken;
+  if (!gate.gave_up_host[dev]) {
+    void* host = nullptr;
+    void* devp = nullptr;
+    if (hipHostMalloc(&host, 64, hipHostMallocMapped) != hipSuccess || hipHostGetDevicePointer(&devp, host, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      return kResidentNotTaken;  // without a way to report a give-up the path is not taken
+    }
+    *static_cast<volatile uint32_t*>(host) = 0u;
+    gate.gave_up_host[dev] = static_cast<volatile uint32_t*>(host);
+    gate.gave_up_dev[dev] = static_cast<uint32_t*>(devp);
+  }
+  uint64_t* phase_log = gate.phase_log.load(std::memory_order_relaxed);
+  if (phase_log && gate.phase_log_bytes.load(std::memory_order_relaxed) < (size_t)grid * 32) phase_log = nullptr;
   if (gate.used[dev] && gate.last_stream[dev] != stream) {
     // mark the tail of the stream that ran the previous resident kernel and wait for it here
     if (!gate.event[dev] && hipEventCreateWithFlags(&gate.event[dev], hipEventDisableTiming) != hipSuccess) {
@@ -377,7 +447,7 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
     }
   }
   kernel<<<(unsigned)grid, kBlock, kResLdsBytes, stream>>>(x, nvec, tail, w, o, o2, amax_out, scale_out, fmax0, fmax1,
-                                                         spin_limit);
+                                                         spin_limit, gate.gave_up_dev[dev], phase_log);
   const int st = launch_status();
   if (st == DT_OK) {
     gate.used[dev] = true;
@@ -394,6 +464,12 @@ inline int launch_resident(const void* x, int in_dtype, int64_t numel, int out_d
   // of the 256 MiB last-level cache faster than this kernel's barrier costs (32 MiB bf16: 17.0 vs
   // 18.4 us).  Below, one launch beats two; above, the second read goes to HBM (128 MiB: 50 vs 61 us).
   const int64_t bytes = numel * (in_dtype == DT_F32 ? 4 : 2);
+  // An earlier launch of the one-kernel path on this device gave up waiting for the whole chip (its
+  // outputs are NaN): say so once, and leave the path off for the rest of the process.
+  if (resident_take_gave_up()) {
+    (void)dt_set_tuning("dynamic.resident", 0);
+    return DT_ERR_RESIDENT_GAVE_UP;
+  }
   if (!tuning("dynamic.resident") || bytes < (int64_t)tuning("dynamic.resident_min_kib") * 1024) return kResidentNotTaken;
   if (bytes >= (int64_t)tuning("dynamic.resident_gap_lo_kib") * 1024 && bytes < (int64_t)tuning("dynamic.resident_gap_hi_kib") * 1024)
     return kResidentNotTaken;

@@ -3,8 +3,10 @@
  *
  * Plain pointers and sizes only: no torch types, no C++ types, no exceptions.  Every entry
  * point validates its arguments on the host, enqueues its kernels on `stream` (NULL = the
- * legacy default stream), never synchronises, never allocates, and returns a dt_status
- * code.  All data pointers are device pointers on the current HIP device.
+ * legacy default stream), never synchronises, never allocates device memory, and returns a
+ * dt_status code.  (One exception to "never allocates": the first per-tensor dynamic quantization
+ * that takes the one-kernel path on a device makes one 64-byte block of pinned HOST memory and keeps
+ * it, see dt_dynamic_scaled_quant.)  All data pointers are device pointers on the current HIP device.
  *
  * Each declaration cites the reference (drisspg/driss_torch) interface it stands in for;
  * paths are relative to the reference tree.  The torch-facing registration shim
@@ -35,7 +37,10 @@ enum dt_status {
   DT_ERR_WORKSPACE = 5,       /* workspace missing or too small */
   DT_ERR_INVALID_MODE = 6,    /* round_mode / axis / layout code out of range */
   DT_ERR_LAUNCH = 7,          /* hipGetLastError() after the launch was not hipSuccess */
-  DT_ERR_EMPTY = 8            /* reduction over zero elements */
+  DT_ERR_EMPTY = 8,           /* reduction over zero elements */
+  DT_ERR_RESIDENT_GAVE_UP = 9 /* an EARLIER per-tensor dynamic quantization on this device gave up waiting for
+                                 the whole chip and wrote NaN outputs (see dt_dynamic_scaled_quant); nothing
+                                 was launched by this call; the one-kernel path is off from now on */
 };
 
 /* element types of the high-precision operand */
@@ -97,7 +102,22 @@ DT_API int dt_saturated_cast(const void* x, int in_dtype, int64_t numel, const f
  * src/dynamic_scaled_quant.cu:157-176 (host), :119-153 (launch), :83-118 (kernel); the
  * scale formula is the one its test checks, test/test_dynamic_quant.py:36 (the kernel's
  * own `fmax / (amax + 1e-12)` at :111 differs in the last bits).  amax_out / scale_out may
- * be NULL.  The reference runs fp32 input only (:130,135); bf16 is accepted here.        */
+ * be NULL.  The reference runs fp32 input only (:130,135); bf16 is accepted here.
+ *
+ * A tensor that fits the chip (128 MiB on 256 CUs, up to 4 x that partly) is quantized by ONE kernel
+ * that occupies every CU and waits inside for all of its workgroups, where the reference uses a
+ * cooperative launch (:144-150).  That assumes THIS PROCESS OWNS THE GPU: the library chains such
+ * launches of one process, and avoids streams with a CU mask, processes with a CU mask in the
+ * environment and streams under graph capture, but it cannot see another process.  If the chip is
+ * not free within a bounded wait ("dynamic.resident_spin_limit"), the waiting workgroups give up:
+ * their outputs, amax and scale are NaN, every kernel still runs to its end, a word of pinned host
+ * memory is set, and the NEXT dt_dynamic_scaled_quant / _pair call on that device launches nothing,
+ * returns DT_ERR_RESIDENT_GAVE_UP once and switches the one-kernel path off for the process
+ * (dt_set_tuning("dynamic.resident", 0); calls after that take the two kernels).  The workspace stays
+ * usable.  dt_dynamic_quant_gave_up() asks the same question without a quantization call: 1 if a
+ * completed launch on the current device gave up since the last time it was asked (and clears it).
+ * dt_set_tuning("dynamic.resident", 0) up front avoids the one-kernel path altogether.            */
+DT_API int dt_dynamic_quant_gave_up(void);
 DT_API int dt_dynamic_scaled_quant(const void* x, int in_dtype, int64_t numel, int out_dtype,
                                    int round_mode, void* out, float* amax_out, float* scale_out,
                                    void* workspace, size_t workspace_bytes, dt_stream_t stream);
@@ -232,6 +252,12 @@ DT_API int dt_mx_fp4_bf16_ws(const void* a, const void* b, const uint8_t* sfa, c
  * or DT_ERR_INVALID_MODE for an unknown key.  Not part of the reference's surface.        */
 DT_API int dt_set_tuning(const char* key, int value);
 DT_API int dt_get_tuning(const char* key, int* value);
+
+/* Benchmarking aid, no counterpart in the reference: while a device buffer is set here (8-byte aligned,
+ * at least 32 bytes per CU; NULL switches it off), every one-kernel dynamic quantization writes four
+ * readings of the 100 MHz constant-rate counter per workgroup into it (uint64[workgroup][4]: start,
+ * share loaded and reduced, released from the grid barrier, stores done).                          */
+DT_API int dt_set_phase_log(void* device_buffer, size_t bytes);
 
 #ifdef __cplusplus
 }

@@ -416,8 +416,10 @@ def test_mx_gemm_argument_errors(d):
 
 
 def test_mx_gemm_config5_full_size(d):
-    """8192^3 from the row-wise cast of N(0,1) operands, scales written blocked by the cast
-    itself; checked on sampled rows against the float64 dequantized product."""
+    """8192^3 from the row-wise cast of N(0,1) operands, scales written blocked by the cast itself
+    (1024 tiles of 256 x 256: four whole rounds of the chip).  Every entry of the output against the
+    fp32 product of the dequantized operands, computed on the device (a library matmul is the
+    reference), and sampled rows against the float64 product on the host."""
     M = N = K = 8192
     a = util.normal((M, K), 1005).cuda()
     b = util.normal((N, K), 1006).cuda()
@@ -426,6 +428,26 @@ def test_mx_gemm_config5_full_size(d):
     out = d.mx_fp8_bf16(a_data, b_data.t(), sa, sb)
     _, a_plain = d.mx_fp8_quantize(a)
     _, b_plain = d.mx_fp8_quantize(b)
+    del a, b
+
+    def dequant(data, scale, rows):
+        s = torch.exp2(scale.view(torch.uint8).view(rows, K // 32).float() - 127.0).repeat_interleave(32, dim=1)
+        return data.float() * s
+
+    dga, dgb = dequant(a_data, a_plain, M), dequant(b_data, b_plain, N)
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        ref32 = dga @ dgb.T
+        bound32 = dga.abs() @ dgb.abs().T
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+    del dga, dgb
+    err = (out.float() - ref32).abs()
+    assert bool((err <= bound32 * 2**-8 + 1e-30).all()), f"max rel {(err / bound32).max().item():.3e}"
+    sqnr_all = 20 * torch.log10(torch.norm(ref32) / torch.norm(out.float() - ref32))
+    assert sqnr_all.item() > 50, sqnr_all.item()
+    del err, ref32, bound32
     rows = torch.tensor([0, 1, 127, 128, 4095, 4096, 5000, 8191])
     da = eager.mx_dequant(a_data[rows.cuda()].cpu(), util.codes(a_plain).view(M, K // 32)[rows])
     db = eager.mx_dequant(b_data.cpu(), util.codes(b_plain).view(N, K // 32))

@@ -223,22 +223,63 @@ def test_resident_not_taken_on_a_stream_restricted_to_some_cus(cabi):
 
 def test_resident_wait_gives_up_loudly(cabi):
     """with a spin limit of one poll most workgroups stop waiting before the last one has arrived:
-    every wave still runs to the end, the sticky flag is set and those workgroups write NaN"""
+    every wave still runs to the end, the sticky flag is set and those workgroups write NaN -- and
+    the caller is told: the next call on the device returns DT_ERR_RESIDENT_GAVE_UP (a RuntimeError
+    through the torch op) and launches nothing, the one-kernel path is off from then on, and the
+    workspace is still good for the two kernels and, once switched on again, for the one."""
+    import driss_torch_amd as d
+
+    L = cabi.lib()
+    assert L.dt_dynamic_quant_gave_up() == 0
     cabi.set_tuning("dynamic.resident", 1)
     cabi.set_tuning("dynamic.resident_spin_limit", 1)
     x = util.normal((8192, 2048), 3).cuda()
-    out, amax, scale = cabi.dynamic_scaled_quant(x, E4, 2)
-    torch.cuda.synchronize()
-    assert _timeout_flag(cabi) == 1
-    codes = util.codes(out)
-    assert ((codes & 0x7F) == 0x7F).any()
-    # re-initialise the workspace (clears the flag) and check that the next call is right again
-    cabi.set_tuning("dynamic.resident_spin_limit", 1 << 19)
-    ws = cabi.workspace(torch.device("cuda"))
-    assert cabi.lib().dt_workspace_init(ws.data_ptr(), ws.numel(), None) == 0
-    torch.cuda.synchronize()
-    out, amax, scale = cabi.dynamic_scaled_quant(x, E4, 2)
     ref, ramax, _ = co.dynamic_scaled_quant(x.cpu(), E4, co.ROUND_V2)
+    try:
+        out, amax, scale = cabi.dynamic_scaled_quant(x, E4, 2)
+        torch.cuda.synchronize()
+        assert _timeout_flag(cabi) == 1
+        codes = util.codes(out)
+        assert ((codes & 0x7F) == 0x7F).any()
+        cabi.set_tuning("dynamic.resident_spin_limit", 1 << 19)
+        # the following call, through the torch op: an error, nothing launched, the path switched off
+        with pytest.raises(RuntimeError, match="gave up"):
+            d.dynamic_scaled_quant(x, E4)
+        assert cabi.get_tuning("dynamic.resident") == 0
+        assert L.dt_dynamic_quant_gave_up() == 0  # reported once
+        # calls after that take the two kernels, on the same workspace, and are right
+        out, amax, scale = cabi.dynamic_scaled_quant(x, E4, 2)
+        assert torch.equal(util.codes(out), ref) and amax.item() == ramax.item()
+        assert torch.equal(util.codes(d.dynamic_scaled_quant(x, E4)), ref)
+        # and so is the one kernel once it is switched on again: the barrier's words were re-armed by the
+        # last workgroup to leave, give-up or not (only the sticky flag stays until dt_workspace_init)
+        cabi.set_tuning("dynamic.resident", 1)
+        out, amax, scale = cabi.dynamic_scaled_quant(x, E4, 2)
+        assert torch.equal(util.codes(out), ref) and amax.item() == ramax.item()
+        assert _timeout_flag(cabi) == 1
+        # the same through the C ABI: give up again, ask without a quantization call
+        cabi.set_tuning("dynamic.resident_spin_limit", 1)
+        cabi.dynamic_scaled_quant(x, E4, 2)
+        torch.cuda.synchronize()
+        cabi.set_tuning("dynamic.resident_spin_limit", 1 << 19)
+        assert L.dt_dynamic_quant_gave_up() == 1 and L.dt_dynamic_quant_gave_up() == 0
+        cabi.dynamic_scaled_quant(x, E4, 2)
+        torch.cuda.synchronize()
+        cabi.set_tuning("dynamic.resident_spin_limit", 1)
+        cabi.dynamic_scaled_quant(x, E4, 2)
+        torch.cuda.synchronize()
+        cabi.set_tuning("dynamic.resident_spin_limit", 1 << 19)
+        with pytest.raises(cabi.DtError) as err:
+            cabi.dynamic_scaled_quant_pair(x, 2)
+        assert err.value.status == 9
+    finally:
+        cabi.set_tuning("dynamic.resident_spin_limit", 1 << 19)
+        cabi.set_tuning("dynamic.resident", 1)
+        L.dt_dynamic_quant_gave_up()
+        ws = cabi.workspace(torch.device("cuda"))
+        assert L.dt_workspace_init(ws.data_ptr(), ws.numel(), None) == 0
+        torch.cuda.synchronize()
+    out, amax, scale = cabi.dynamic_scaled_quant(x, E4, 2)
     assert torch.equal(util.codes(out), ref) and amax.item() == ramax.item()
     assert _timeout_flag(cabi) == 0
 
