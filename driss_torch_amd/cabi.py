@@ -32,6 +32,7 @@ SIGNATURES = {
     "dt_amax": (_i32, [_vp, _i32, _i64, _vp, _vp, _sz, _vp]),
     "dt_saturated_cast": (_i32, [_vp, _i32, _i64, _vp, _i32, _i32, _vp, _vp]),
     "dt_dynamic_scaled_quant": (_i32, [_vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "dt_dynamic_scaled_quant_noalloc": (_i32, [_vp, _i32, _i64, _i32, _i32, _vp, _vp, _vp, _vp]),
     "dt_dynamic_scaled_quant_pair": (_i32, [_vp, _i32, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "dt_amax_scales": (_i32, [_vp, _i32, _i64, _vp, _vp, _vp, _sz, _vp]),
     "dt_saturated_cast_pair": (_i32, [_vp, _i32, _i64, _vp, _i32, _vp, _vp, _vp]),

@@ -101,6 +101,7 @@ const char* dt_status_string(int status) {
     case DT_ERR_RESIDENT_GAVE_UP:
       return "an earlier dynamic quantization on this device gave up waiting for the whole chip and wrote NaN "
              "(is another process using the GPU?); the one-kernel path is now off for this process";
+    case DT_ERR_TOO_LARGE: return "more elements than the no-allocation entry point takes (DT_NOALLOC_MAX_NUMEL)";
     default: return "unknown status";
   }
 }

@@ -9,8 +9,44 @@
 #include "resident_kernels.hpp"
 #include "rowwise_kernels.hpp"
 
+#include <mutex>
+
 namespace {
 inline float fmax_of(int out_dtype) { return out_dtype == DT_E5M2 ? 57344.0f : 448.0f; }
+
+// ---- the reduction workspace of dt_dynamic_scaled_quant_noalloc: device memory that belongs to the
+// library's code object, so that the caller neither allocates nor passes one.  Each device the library
+// runs on holds its own copy at its own address until the process ends; host code never uses the
+// array's name as an address, only what hipGetSymbolAddress returned for the device at hand.
+static __device__ __align__(256) uint8_t scratch[dt::kWsBytes];
+
+constexpr int kScratchDevices = 16;
+std::mutex g_scratch_mu;
+uint8_t* g_scratch_ptr[kScratchDevices] = {};  // per device, looked up at the entry point's first call there
+
+// nullptr with *status set when the lookup fails
+uint8_t* scratch_of_current_device(int* status) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kScratchDevices) {
+    (void)hipGetLastError();
+    *status = DT_ERR_LAUNCH;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+      (void)hipGetLastError();
+      *status = DT_ERR_LAUNCH;
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = static_cast<uint8_t*>(p);
+  }
+  return g_scratch_ptr[dev];
+}
+
+// the words a reduction expects to find zero (a fill kernel, not hipMemsetAsync: callers may capture)
+__global__ void clear_scratch_kernel(uint32_t* p) { p[threadIdx.x] = 0u; }
 }  // namespace
 
 extern "C" int dt_dynamic_scaled_quant(const void* x, int in_dtype, int64_t numel, int out_dtype, int round_mode,
@@ -29,6 +65,27 @@ extern "C" int dt_dynamic_scaled_quant(const void* x, int in_dtype, int64_t nume
   if (st) return st;
   const float* scale = reinterpret_cast<const float*>(static_cast<const uint8_t*>(workspace) + dt::kWsScale);
   return dt::launch_cast<false>(x, in_dtype, numel, scale, out_dtype, round_mode, out, nullptr, s);
+}
+
+extern "C" int dt_dynamic_scaled_quant_noalloc(const void* x, int in_dtype, int64_t numel, int out_dtype, int round_mode,
+                                               void* out, float* amax_out, float* scale_out, dt_stream_t stream) {
+  if (int st = dt::check_cast_args(x, in_dtype, numel, out_dtype, round_mode, out)) return st;
+  if (numel == 0) return DT_ERR_EMPTY;
+  if (numel > DT_NOALLOC_MAX_NUMEL) return DT_ERR_TOO_LARGE;
+  int st = DT_OK;
+  uint8_t* const ws = scratch_of_current_device(&st);
+  if (!ws) return st;
+  hipStream_t s = dt::as_hip(stream);
+  // The array keeps whatever the last call on this device left in it.  A completed call leaves its
+  // counters at zero, but one that was cut short would not: start from zero every time.
+  clear_scratch_kernel<<<1, 128, 0, s>>>(reinterpret_cast<uint32_t*>(ws));
+  if (int e = dt::launch_status()) return e;
+  const float fm = fmax_of(out_dtype);
+  st = in_dtype == DT_F32 ? dt::launch_amax<DT_F32>(x, numel, ws, amax_out, scale_out, 1, fm, 0.f, s)
+                          : dt::launch_amax<DT_BF16>(x, numel, ws, amax_out, scale_out, 1, fm, 0.f, s);
+  if (st) return st;
+  return dt::launch_cast<false>(x, in_dtype, numel, reinterpret_cast<const float*>(ws + dt::kWsScale), out_dtype, round_mode,
+                                out, nullptr, s);
 }
 
 extern "C" int dt_amax_scales(const void* x, int in_dtype, int64_t numel, float* amax_out, float* scale_out,

@@ -38,9 +38,10 @@ enum dt_status {
   DT_ERR_INVALID_MODE = 6,    /* round_mode / axis / layout code out of range */
   DT_ERR_LAUNCH = 7,          /* hipGetLastError() after the launch was not hipSuccess */
   DT_ERR_EMPTY = 8,           /* reduction over zero elements */
-  DT_ERR_RESIDENT_GAVE_UP = 9 /* an EARLIER per-tensor dynamic quantization on this device gave up waiting for
+  DT_ERR_RESIDENT_GAVE_UP = 9,/* an EARLIER per-tensor dynamic quantization on this device gave up waiting for
                                  the whole chip and wrote NaN outputs (see dt_dynamic_scaled_quant); nothing
                                  was launched by this call; the one-kernel path is off from now on */
+  DT_ERR_TOO_LARGE = 10       /* more elements than dt_dynamic_scaled_quant_noalloc takes (DT_NOALLOC_MAX_NUMEL) */
 };
 
 /* element types of the high-precision operand */
@@ -121,6 +122,24 @@ DT_API int dt_dynamic_quant_gave_up(void);
 DT_API int dt_dynamic_scaled_quant(const void* x, int in_dtype, int64_t numel, int out_dtype,
                                    int round_mode, void* out, float* amax_out, float* scale_out,
                                    void* workspace, size_t workspace_bytes, dt_stream_t stream);
+
+/* dt_dynamic_scaled_quant for callers that can neither allocate device memory nor keep a workspace
+ * around: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
+ * no counterpart in the reference (whose op takes its scratch from the caching allocator on every
+ * call, src/dynamic_scaled_quant.cu:172).  Same arguments and the same bits as
+ * dt_dynamic_scaled_quant, without the workspace: the reduction's 4 KiB of scratch live in a device
+ * array that is part of the library itself (one copy per GPU, held until the process ends).  The call
+ * allocates and frees nothing -- no hipMalloc / hipFree, no pinned host memory -- and always runs as the
+ * reduction kernel followed by the cast kernel (never the one-kernel path, which makes a block of host
+ * memory at its first use and is refused under capture anyway); a small fill kernel clears the scratch's
+ * counters first.  At most DT_NOALLOC_MAX_NUMEL elements, else DT_ERR_TOO_LARGE.  All calls on one GPU
+ * share that GPU's array: calls that may overlap there (two streams, two threads) race on it and must
+ * be ordered by the caller; use dt_dynamic_scaled_quant with a workspace per stream for those.  The
+ * first call on a device looks the array's address up (hipGetSymbolAddress): make it outside a capture. */
+#define DT_NOALLOC_MAX_NUMEL ((int64_t)1 << 34)
+DT_API int dt_dynamic_scaled_quant_noalloc(const void* x, int in_dtype, int64_t numel, int out_dtype,
+                                           int round_mode, void* out, float* amax_out, float* scale_out,
+                                           dt_stream_t stream);
 
 /* As above with two outputs from one read of x for the cast: e4m3fn with scale 448/amax and
  * e5m2 with scale 57344/amax.  scale_out, if given, receives {scale_e4m3fn, scale_e5m2}.
