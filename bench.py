@@ -162,7 +162,13 @@ def main():
     step_us = time_launches(step, ns, K, 0)
     step_gbs = step_bytes / (step_us * 1e-6) / 1e9
 
-    phases = resident_phases(torch, cabi, step, ns) if args.phases else None
+    phases = None
+    if args.phases:
+        phases = {"resident_quant_kernel (the step)": kernel_phases(
+            torch, cabi, step, ["load and reduce", "grid barrier", "convert and store"])}
+        amax_tmp = torch.empty(1, dtype=torch.float32, device=dev)
+        phases["amax_kernel, bf16 [8192,8192]"] = kernel_phases(
+            torch, cabi, lambda i: cabi.amax(xs[i % ns], amax_tmp), ["load", "workgroup reduce", "atomics"])
 
     # for comparison: the two-kernel path every larger tensor takes (amax, then cast), the cast
     # bracketed by an event pair per launch (adds about 4 us of dispatch latency to it)
@@ -215,7 +221,7 @@ def main():
                             "cast_kernel(pair) traffic": cast_traffic},
     }
     if phases:
-        result["resident_phases"] = phases
+        result["phases"] = phases
     if args.calibrate_copy:
         src = xs[0]
         dst = torch.empty_like(src)
@@ -233,20 +239,20 @@ def main():
     print(json.dumps(result))
 
 
-def resident_phases(torch, cabi, step, ns, launches=20):
-    """Where the step's one kernel spends its time: every workgroup writes four readings of the 100 MHz
-    constant-rate counter (start, share loaded and reduced, released from the grid barrier, stores
-    done; dt_set_phase_log), collected here over `launches` launches with a synchronisation after each.
-    All figures in microseconds, medians over the launches; t = 0 is the first workgroup's start."""
+def kernel_phases(torch, cabi, launch, names, launches=20):
+    """Where a kernel spends its time: with a phase log set (dt_set_phase_log) every workgroup of the
+    one-kernel dynamic quantization and of the amax reduction writes four readings of the 100 MHz
+    constant-rate counter (start and three phase ends, `names`), collected here over `launches`
+    launches of `launch(i)` with a synchronisation after each.  All figures in microseconds, medians
+    over the launches; t = 0 is the first workgroup's start."""
     L = cabi.lib()
-    cus = torch.cuda.get_device_properties(0).multi_processor_count
-    log = torch.zeros((cus, 4), dtype=torch.int64, device="cuda")
+    log = torch.zeros((1024, 4), dtype=torch.int64, device="cuda")
     assert L.dt_set_phase_log(log.data_ptr(), log.numel() * 8) == 0
     rows = []
     try:
         for i in range(launches + 3):
             log.zero_()
-            step(i % ns)
+            launch(i)
             torch.cuda.synchronize()
             t = log.cpu().double()
             t = t[t[:, 0] > 0]  # workgroups of the grid
@@ -254,25 +260,26 @@ def resident_phases(torch, cabi, step, ns, launches=20):
                 continue
             t = (t - t[:, 0].min()) / 100.0  # 100 MHz -> us
             med = lambda v: float(v.median())  # noqa: E731
-            rows.append({
-                "workgroups": int(t.shape[0]),
-                "last_workgroup_starts_at": float(t[:, 0].max()),
-                "load_and_reduce_per_workgroup_median": med(t[:, 1] - t[:, 0]),
-                "first_workgroup_loaded_at": float(t[:, 1].min()),
-                "last_workgroup_loaded_at": float(t[:, 1].max()),
-                "released_at_median": med(t[:, 2]),
-                "released_at_last": float(t[:, 2].max()),
-                "wait_in_barrier_per_workgroup_median": med(t[:, 2] - t[:, 1]),
-                "release_after_last_arrival_median": med(t[:, 2]) - float(t[:, 1].max()),
-                "convert_and_store_per_workgroup_median": med(t[:, 3] - t[:, 2]),
-                "first_workgroup_done_at": float(t[:, 3].min()),
-                "last_workgroup_done_at": float(t[:, 3].max()),
-            })
+            row = {"workgroups": int(t.shape[0]), "last_workgroup_starts_at": float(t[:, 0].max())}
+            for k, name in enumerate(names, start=1):
+                row[f"{name}: per workgroup, median"] = med(t[:, k] - t[:, k - 1])
+                row[f"{name}: first workgroup done at"] = float(t[:, k].min())
+                row[f"{name}: median workgroup done at"] = med(t[:, k])
+                row[f"{name}: last workgroup done at"] = float(t[:, k].max())
+            # by XCD (workgroup b runs on XCD b % 8): when each XCD's slowest workgroup is done with everything
+            if t.shape[0] % 8 == 0:
+                row["last phase done at, slowest workgroup of each XCD"] = [float(t[x::8, 3].max()) for x in range(8)]
+            rows.append(row)
     finally:
         L.dt_set_phase_log(None, 0)
     if not rows:
         return None
-    out = {k: round(statistics.median(r[k] for r in rows), 2) for k in rows[0]}
+    out = {}
+    for k in rows[0]:
+        if isinstance(rows[0][k], list):
+            out[k] = [round(statistics.median(r[k][x] for r in rows), 2) for x in range(len(rows[0][k]))]
+        else:
+            out[k] = round(statistics.median(r[k] for r in rows), 2)
     out["launches"] = len(rows)
     out["unit"] = "us (100 MHz counter, 0.01 us resolution)"
     return out
@@ -322,13 +329,14 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False):
         hbm_row("saturated_cast", "fp32 [8192,8192] -> e4m3fn", n * 5,
                 lambda i: (rnd((8192, 8192), f32, i), torch.empty((8192, 8192), dtype=e4, device=dev)),
                 lambda x, o: cabi.saturated_cast(x, scale1, e4, cabi.ROUND_F32, o))
-        hbm_row("dynamic_scaled_quant (one resident kernel)", "bf16 [8192,8192] -> amax, scale, e4m3fn", n * 5,
+        # bytes of the dynamic rows: what the kernel must move (x once for the part the chip holds)
+        hbm_row("dynamic_scaled_quant (one resident kernel)", "bf16 [8192,8192] -> amax, scale, e4m3fn", n * 3,
                 lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 8192), dtype=e4, device=dev),
                            torch.empty(1, device=dev), torch.empty(1, device=dev)),
                 lambda x, o, a, s_: cabi.dynamic_scaled_quant(x, e4, cabi.ROUND_BF16_SCALE_PRODUCT, o, a, s_))
         # twice what the chip holds: 128 MiB stays in registers and LDS, the other 128 MiB is read twice
         n2 = 16384 * 8192
-        hbm_row("dynamic_scaled_quant pair, 2 x the chip's capacity", "bf16 [16384,8192] -> amax, scales, e4m3fn and e5m2", n2 * 6,
+        hbm_row("dynamic_scaled_quant pair, 2 x the chip's capacity", "bf16 [16384,8192] -> amax, scales, e4m3fn and e5m2", n2 * 5,
                 lambda i: (rnd((16384, 8192), bf16, i), torch.empty((16384, 8192), dtype=e4, device=dev),
                            torch.empty((16384, 8192), dtype=e5, device=dev), torch.empty(1, device=dev), torch.empty(2, device=dev)),
                 lambda x, o4, o5, a, s_: cabi.dynamic_scaled_quant_pair(x, cabi.ROUND_BF16_SCALE_PRODUCT, o4, o5, a, s_))

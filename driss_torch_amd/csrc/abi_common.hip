@@ -35,8 +35,8 @@ struct Knob {
 Knob g_knobs[] = {
     {"amax.blocks_per_cu", 1},
     {"amax.stream_before_cast", 0},
-    {"cast.blocks_per_cu", 2},
-    {"cast.pair_blocks_per_cu", 2},
+    {"cast.blocks_per_cu", 1},
+    {"cast.pair_blocks_per_cu", 1},
     {"rowwise.block_from_vecs", 257},
     {"mx.blocks_per_cu", 32},
     {"mx.col_blocks_per_cu", 32},
@@ -55,6 +55,9 @@ Knob g_knobs[] = {
 };
 constexpr int kNumKnobs = sizeof(g_knobs) / sizeof(g_knobs[0]);
 
+std::atomic<uint64_t*> g_phase_log{nullptr};
+std::atomic<size_t> g_phase_log_bytes{0};
+
 constexpr int kMaxDevices = 16;
 DeviceFacts g_facts[kMaxDevices];
 std::once_flag g_facts_once[kMaxDevices];
@@ -64,6 +67,11 @@ int tuning(const char* key) {
   for (int i = 0; i < kNumKnobs; ++i)
     if (strcmp(g_knobs[i].key, key) == 0) return g_knobs[i].value.load(std::memory_order_relaxed);
   return 0;
+}
+
+uint64_t* phase_log(size_t need_bytes) {
+  uint64_t* p = g_phase_log.load(std::memory_order_relaxed);
+  return p && g_phase_log_bytes.load(std::memory_order_relaxed) >= need_bytes ? p : nullptr;
 }
 
 const DeviceFacts& device_facts() {
@@ -115,8 +123,15 @@ int dt_workspace_init(void* workspace, size_t workspace_bytes, dt_stream_t strea
   if (workspace_bytes < dt::kWsBytes) return DT_ERR_WORKSPACE;
   if (!dt::aligned(workspace, 256)) return DT_ERR_MISALIGNED;
   // a fill kernel rather than hipMemsetAsync, so the call is safe under graph capture
-  dt::zero_words_kernel<<<1, 128, 0, dt::as_hip(stream)>>>(static_cast<uint32_t*>(workspace), 128);
+  dt::zero_words_kernel<<<dt::kWsBytes / 4 / 256, 256, 0, dt::as_hip(stream)>>>(static_cast<uint32_t*>(workspace), dt::kWsBytes / 4);
   return dt::launch_status();
+}
+
+int dt_set_phase_log(void* device_buffer, size_t bytes) {
+  if (device_buffer && !dt::aligned(device_buffer, 8)) return DT_ERR_MISALIGNED;
+  dt::g_phase_log_bytes.store(device_buffer ? bytes : 0, std::memory_order_relaxed);
+  dt::g_phase_log.store(static_cast<uint64_t*>(device_buffer), std::memory_order_relaxed);
+  return DT_OK;
 }
 
 int dt_set_tuning(const char* key, int value) {

@@ -24,6 +24,10 @@ const DeviceFacts& device_facts();  // of the current device, cached per device
 
 int tuning(const char* key);  // current value of a launch knob
 
+// Device buffer for per-workgroup clock readings (dt_set_phase_log), or null when none is set or it
+// holds fewer than `need_bytes`.
+uint64_t* phase_log(size_t need_bytes);
+
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 inline int64_t ceil_div(int64_t a, int64_t b) { return a / b + (a % b != 0); }  // src/include/utils.h:37-39
 

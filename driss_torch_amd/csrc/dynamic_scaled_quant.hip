@@ -139,11 +139,3 @@ extern "C" int dt_dynamic_scaled_quant_rowwise(const void* x, int in_dtype, int6
 }
 
 extern "C" int dt_dynamic_quant_gave_up(void) { return dt::resident_take_gave_up() ? 1 : 0; }
-
-extern "C" int dt_set_phase_log(void* device_buffer, size_t bytes) {
-  if (device_buffer && !dt::aligned(device_buffer, 8)) return DT_ERR_MISALIGNED;
-  dt::ResidentGate& gate = dt::resident_gate();
-  gate.phase_log_bytes.store(device_buffer ? bytes : 0, std::memory_order_relaxed);
-  gate.phase_log.store(static_cast<uint64_t*>(device_buffer), std::memory_order_relaxed);
-  return DT_OK;
-}

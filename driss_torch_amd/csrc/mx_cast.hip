@@ -18,8 +18,8 @@ int launch_mx(const MxArgs& a) {
   constexpr int kV = InTraits<IN>::kVec;
   const int64_t numel = a.rows * a.cols, nblocks = numel / 32;
   const int cus = device_facts().cu_count;
-  const bool x_vec = aligned(a.x, 16);
-  if (a.axis == 1 && !a.transpose && x_vec && aligned(a.data, 8) && nblocks < (1ll << 28)) {
+  // x only has to be aligned to its element: the kernels load it through element-aligned vector types
+  if (a.axis == 1 && !a.transpose && aligned(a.data, 8) && nblocks < (1ll << 28)) {
     const int64_t nsuper = ceil_div(nblocks, 64);
     int64_t waves = (int64_t)cus * tuning("mx.blocks_per_cu") * (kBlock / kWave);
     if (waves > nsuper) waves = nsuper;
@@ -35,20 +35,10 @@ int launch_mx(const MxArgs& a) {
                                                                  a.data, a.scale);
     return launch_status();
   }
-  // the same for an x that starts off a 16-byte boundary (a view): element-aligned vector loads
-  if (a.axis == 1 && !a.transpose && !x_vec && aligned(a.data, 8) && nblocks < (1ll << 28)) {
-    const int64_t nsuper = ceil_div(nblocks, 64);
-    int64_t waves = (int64_t)cus * tuning("mx.blocks_per_cu") * (kBlock / kWave);
-    if (waves > nsuper) waves = nsuper;
-    const unsigned grid = (unsigned)ceil_div(waves, kBlock / kWave);
-    mx_row_kernel<IN, OUT, LAYOUT, false, true><<<grid, kBlock, 0, a.stream>>>(a.x, (uint32_t)nblocks, (uint32_t)(a.cols / 32),
-                                                                              a.data, a.scale);
-    return launch_status();
-  }
   // Transposed column cast: the one-read kernel without its row-wise half (16-byte loads, half-wave
   // row split) wherever a lane's kV columns are whole; 8192 x 8192 bf16 38.3 vs 40.2 us for
   // mx_col_t_kernel, 16384 x 4096 36.3 vs 41.0 us.  Tile order by shape, as for the full kernel.
-  if (a.axis == 0 && a.transpose && x_vec && a.cols % kV == 0 && aligned(a.data, 16) && aligned(a.scale, 4) &&
+  if (a.axis == 0 && a.transpose && a.cols % kV == 0 && aligned(a.data, 16) && aligned(a.scale, 4) &&
       a.rows < (1ll << 31) && a.cols < (1ll << 31) && tuning("mx.colt_via_dual")) {
     constexpr int kTileCols = 32 * kV;
     const int64_t tiles = ceil_div(a.rows, (int64_t)kDualRows) * ceil_div(a.cols, (int64_t)kTileCols);
@@ -58,8 +48,8 @@ int launch_mx(const MxArgs& a) {
       return launch_status();
     }
   }
-  if (a.axis == 0 && a.transpose && x_vec && a.cols % 4 == 0 && (a.cols * InTraits<IN>::kBytes) % 16 == 0 &&
-      aligned(a.data, 16) && aligned(a.scale, 4) && a.rows < (1ll << 31) && a.cols < (1ll << 31)) {
+  if (a.axis == 0 && a.transpose && a.cols % 4 == 0 && aligned(a.data, 16) && aligned(a.scale, 4) &&
+      a.rows < (1ll << 31) && a.cols < (1ll << 31)) {
     const int64_t tiles = ceil_div(a.rows, (int64_t)kColTRows) * ceil_div(a.cols, (int64_t)kColTCols);
     if (tiles <= 0x7FFFFFFFll) {
       mx_col_t_kernel<IN, OUT, LAYOUT><<<(unsigned)tiles, kBlock, 0, a.stream>>>(a.x, (uint32_t)a.rows, (uint32_t)a.cols,
@@ -67,7 +57,7 @@ int launch_mx(const MxArgs& a) {
       return launch_status();
     }
   }
-  if (a.axis == 0 && !a.transpose && x_vec && a.cols % kV == 0 && aligned(a.data, 16) && aligned(a.scale, 8) &&
+  if (a.axis == 0 && !a.transpose && a.cols % kV == 0 && aligned(a.data, 16) && aligned(a.scale, 8) &&
       a.rows < (1ll << 31) && a.cols < (1ll << 31) && LAYOUT == DT_SCALE_PLAIN) {
     const int64_t tiles = (a.rows / 32) * ceil_div(a.cols, (int64_t)kWave * kV);
     if (tiles <= 0x7FFFFFFFll) {
@@ -76,6 +66,18 @@ int launch_mx(const MxArgs& a) {
       mx_col_kernel<IN, OUT><<<(unsigned)grid, kBlock, 0, a.stream>>>(a.x, (uint32_t)a.rows, (uint32_t)a.cols, a.data,
                                                                      a.scale, (uint32_t)tiles);
       return launch_status();
+    }
+  }
+  // blocks along the rows with a transposed payload: through the LDS transpose tile
+  if constexpr (LAYOUT == DT_SCALE_PLAIN) {
+    if (a.axis == 1 && a.transpose && a.rows % 16 == 0 && aligned(a.data, 16) && aligned(a.scale, 4) &&
+        a.rows < (1ll << 31) && a.cols < (1ll << 31)) {
+      const int64_t tiles = ceil_div(a.rows, (int64_t)kDualRows) * ceil_div(a.cols, (int64_t)(32 * kV));
+      if (tiles <= 0x7FFFFFFFll) {
+        mx_row_t_kernel<IN, OUT><<<(unsigned)tiles, kBlock, 0, a.stream>>>(a.x, (uint32_t)a.rows, (uint32_t)a.cols, a.data,
+                                                                          a.scale);
+        return launch_status();
+      }
     }
   }
   // general orientation / alignment
@@ -116,7 +118,7 @@ constexpr int kNotTaken = -1;
 template <int IN, int OUT, int LAYOUT>
 int launch_dual(const DualArgs& a) {
   constexpr int kTileCols = 32 * InTraits<IN>::kVec;
-  if (!aligned(a.x, 16) || !aligned(a.data_r, 8) || !aligned(a.data_c, 16) || !aligned(a.scale_r, 4) ||
+  if (!aligned(a.data_r, 8) || !aligned(a.data_c, 16) || !aligned(a.scale_r, 4) ||
       !aligned(a.scale_c, 4) || a.rows >= (1ll << 31) || a.cols >= (1ll << 31))
     return kNotTaken;
   const int64_t tiles = ceil_div(a.rows, (int64_t)kDualRows) * ceil_div(a.cols, (int64_t)kTileCols);

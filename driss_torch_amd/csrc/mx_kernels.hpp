@@ -10,6 +10,7 @@
 //                  are full 128-byte rows of the [cols, rows] output.
 //  mx_dual_kernel  blocks along rows (payload as is) and down columns (payload transposed) from
 //                  one read of the input.
+//  mx_row_t_kernel blocks along rows, payload transposed through the same LDS tile.
 //  mx_any_kernel   one thread per block, arbitrary strides: covers every (axis, transpose)
 //                  pair and shapes the fast kernels do not take.
 #pragma once
@@ -138,6 +139,21 @@ __device__ __forceinline__ uint32_t vec_absmax_bits(u32x4 w) {
   }
 }
 
+// Streaming loads of x through vector types that claim no more than the element's alignment.  The
+// instruction is the same global_load_dwordx4 / dwordx2 ... nt as for an aligned type, and the device
+// serves it at any address (an access that straddles a line costs the second line), so every kernel
+// below takes an x that is only aligned to its element, e.g. a view that starts one element into its
+// buffer (8192 x 8192 bf16 one element off: within a few percent of the aligned case).
+typedef u32x2 u32x2_elem2 __attribute__((aligned(2)));
+template <int IN>
+__device__ __forceinline__ u32x4 ld_x16(const void* p) {
+  typedef typename std::conditional<IN == DT_F32, u32x4_elem4, u32x4_elem2>::type vec_t;
+  return __builtin_nontemporal_load(static_cast<const vec_t*>(p));
+}
+__device__ __forceinline__ u32x2 ld_x8_16bit(const void* p) {
+  return __builtin_nontemporal_load(static_cast<const u32x2_elem2*>(p));
+}
+
 // ------------------------------------------------------------------ blocks along rows
 // The matrix is a flat run of 32-element blocks.  One wave pass ("super-chunk") covers 64
 // blocks as LPB chunks of 64 vectors; lane l ends up holding the scale byte of chunk
@@ -148,9 +164,7 @@ __device__ __forceinline__ uint32_t vec_absmax_bits(u32x4 w) {
 // row -- because those are the scales that sit next to each other in the blocked layout: the 64
 // bytes of a pass then fall into 4 runs of 16 bytes instead of 16 runs of 4, which costs a
 // quarter of the memory transactions (36.8 -> 33 us at 8192 x 8192 bf16).
-// XANY: x is only aligned to its element (a view that starts at an odd element): the same 16-byte
-// loads through a vector type that claims no more (the device serves them).
-template <int IN, int OUT, int LAYOUT, bool BAND4 = false, bool XANY = false>
+template <int IN, int OUT, int LAYOUT, bool BAND4 = false>
 __global__ __launch_bounds__(kBlock) void mx_row_kernel(const void* __restrict__ x, uint32_t nblocks,
                                                         uint32_t kblocks, uint8_t* __restrict__ data,
                                                         uint8_t* __restrict__ scale) {
@@ -184,12 +198,7 @@ __global__ __launch_bounds__(kBlock) void mx_row_kernel(const void* __restrict__
 #pragma unroll
     for (int c = 0; c < LPB; ++c) {
       const uint32_t vi = vec_index(c);
-      if constexpr (XANY) {
-        typedef typename std::conditional<IN == DT_F32, u32x4_elem4, u32x4_elem2>::type vec_t;
-        w[c] = vi < nvec ? reinterpret_cast<const vec_t*>(x)[vi] : u32x4{0u, 0u, 0u, 0u};
-      } else {
-        w[c] = vi < nvec ? ld_stream(v + vi) : u32x4{0u, 0u, 0u, 0u};
-      }
+      w[c] = vi < nvec ? ld_x16<IN>(v + vi) : u32x4{0u, 0u, 0u, 0u};
     }
     uint32_t mybyte = 0;
 #pragma unroll
@@ -270,7 +279,7 @@ __global__ __launch_bounds__(kBlock) void mx_col_kernel(const void* __restrict__
     if (col0 < cols) {
       const uint8_t* p = static_cast<const uint8_t*>(x) + (uint64_t)(tr * 32u + w * 8u) * pitch + (uint64_t)col0 * kB;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = ld_stream(reinterpret_cast<const u32x4*>(p + i * pitch));
+      for (int i = 0; i < 8; ++i) v[i] = ld_x16<IN>(p + i * pitch);
     } else {
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[i] = u32x4{0u, 0u, 0u, 0u};
@@ -407,7 +416,10 @@ __global__ __launch_bounds__(kBlock) void mx_col_t_kernel(const void* __restrict
     uint32_t cm[4] = {0, 0, 0, 0};
     const uint8_t* p = static_cast<const uint8_t*>(x) + ((uint64_t)row0 * cols + col0) * kB;
 #pragma unroll
-    for (int i = 0; i < 32; ++i) wv[i] = ld_stream(reinterpret_cast<const row_t*>(p + (uint64_t)i * cols * kB));
+    for (int i = 0; i < 32; ++i) {
+      if constexpr (IN == DT_F32) wv[i] = ld_x16<IN>(p + (uint64_t)i * cols * kB);
+      else wv[i] = ld_x8_16bit(p + (uint64_t)i * cols * kB);
+    }
     // the word that holds column c of row i (fp32: the element itself; 16-bit: it and its neighbour)
     auto word = [&](int i, int c) -> uint32_t {
       if constexpr (IN == DT_F32) return c == 0 ? wv[i].x : c == 1 ? wv[i].y : c == 2 ? wv[i].z : wv[i].w;
@@ -581,7 +593,7 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
   if (active) {
     const uint8_t* p = static_cast<const uint8_t*>(x) + ((uint64_t)row0 * cols + col0) * kB;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) v[i] = ld_stream(reinterpret_cast<const u32x4*>(p + (uint64_t)i * cols * kB));
+    for (int i = 0; i < 16; ++i) v[i] = ld_x16<IN>(p + (uint64_t)i * cols * kB);
   } else {
 #pragma unroll
     for (int i = 0; i < 16; ++i) v[i] = u32x4{0u, 0u, 0u, 0u};
@@ -708,6 +720,92 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
           if (c + k < KB) scale_r[scale_offset<LAYOUT>(r, c + k, KB)] = (uint8_t)(sw >> (8 * k));
       }
     }
+  }
+}
+
+// ----------------------------------------- blocks along rows, transposed payload
+// (axis 1, transpose): the row-wise cast written as [cols, rows], scales [cols/32, rows].  The
+// geometry of mx_dual_kernel: a workgroup owns 128 rows x 32*kV columns, a lane 16 rows x kV adjacent
+// columns, which lie in one row-direction block.  Row-block maxima over the neighbouring lanes; the
+// payload is converted four rows of one column at a time (four different scales per word) into the
+// same swizzled LDS tile [column][128 rows] and leaves as 128-byte rows; the scale bytes leave as
+// kRowBlocks runs of 128 bytes.  Tiles are numbered down the rows first, so that neighbouring
+// workgroups write adjacent pieces of the same output rows.  rows % 16 == 0.
+template <int IN, int OUT>
+__global__ __launch_bounds__(kBlock) void mx_row_t_kernel(const void* __restrict__ x, uint32_t rows, uint32_t cols,
+                                                          uint8_t* __restrict__ data, uint8_t* __restrict__ scale) {
+  constexpr int kV = InTraits<IN>::kVec;
+  constexpr int kB = InTraits<IN>::kBytes;
+  constexpr int kTileCols = 32 * kV;
+  constexpr int kRowBlocks = kTileCols / 32;
+  constexpr int LPB = 32 / kV;
+  __shared__ __attribute__((aligned(16))) uint8_t tile[kTileCols * kDualPitch];
+  __shared__ __attribute__((aligned(16))) uint8_t rtile[kRowBlocks * kDualRows];  // [block][row]
+  const int tid = threadIdx.x, lane = tid % kWave, w = tid / kWave, h = lane >> 5, c8 = lane & 31;
+  const uint32_t row_tiles = (rows + kDualRows - 1) / kDualRows;
+  const uint32_t tc = blockIdx.x / row_tiles, tr = blockIdx.x - tc * row_tiles;
+  const uint32_t lrow0 = w * 32 + h * 16;
+  const uint32_t row0 = tr * kDualRows + lrow0, col0 = tc * kTileCols + c8 * kV;
+  const bool active = row0 < rows && col0 < cols;  // rows % 16 == 0 and cols % 32 == 0: all of a lane or none
+
+  saturate_fp8_conversions();
+  u32x4 v[16];
+  if (active) {
+    const uint8_t* p = static_cast<const uint8_t*>(x) + ((uint64_t)row0 * cols + col0) * kB;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = ld_x16<IN>(p + (uint64_t)i * cols * kB);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = u32x4{0u, 0u, 0u, 0u};
+  }
+  float sc[16];
+  uint32_t rb[4] = {0u, 0u, 0u, 0u}, nanmask[4] = {0u, 0u, 0u, 0u};  // per row: scale byte, 0xFF where the block holds a NaN
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    uint32_t m = quad_umax(vec_absmax_bits<IN>(v[i]));
+    if constexpr (LPB == 8) m = umax(m, dpp<kDppRowHalfMirror>(m));
+    const MxScale<OUT> s = mx_scale_from_absbits<OUT>(m);
+    sc[i] = s.scale;
+    rb[i / 4] |= s.byte << (8 * (i % 4));
+    nanmask[i / 4] |= s.nan ? (0xFFu << (8 * (i % 4))) : 0u;
+  }
+  auto word = [&](int i, int c) -> uint32_t {
+    const int k = IN == DT_F32 ? c : c / 2;
+    return k == 0 ? v[i].x : k == 1 ? v[i].y : k == 2 ? v[i].z : v[i].w;
+  };
+  const uint32_t chunk = (uint32_t)(w * 2 + h);
+#pragma unroll
+  for (int c = 0; c < kV; ++c) {
+    uint32_t r[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if constexpr (IN == DT_F32)
+        r[q] = cvt_scaled_4x32_each<OUT>(word(4 * q, c), word(4 * q + 1, c), word(4 * q + 2, c), word(4 * q + 3, c), sc + 4 * q);
+      else
+        r[q] = cvt_scaled_4x16_each<IN, OUT>(gather_halves(c & 1, word(4 * q, c), word(4 * q + 1, c)),
+                                             gather_halves(c & 1, word(4 * q + 2, c), word(4 * q + 3, c)), sc + 4 * q);
+      r[q] = (r[q] & ~nanmask[q]) | (0x7F7F7F7Fu & nanmask[q]);
+    }
+    const uint32_t col = (uint32_t)(c8 * kV + c);
+    *reinterpret_cast<u32x4*>(tile + col * kDualPitch + ((chunk ^ ((col >> 4) & 7u)) << 4)) = u32x4{r[0], r[1], r[2], r[3]};
+  }
+  if ((c8 % LPB) == 0) *reinterpret_cast<u32x4*>(rtile + (c8 / LPB) * kDualRows + lrow0) = u32x4{rb[0], rb[1], rb[2], rb[3]};
+  __syncthreads();
+
+  const uint32_t trow0 = tr * kDualRows, tcol0 = tc * kTileCols;
+#pragma unroll
+  for (int i = 0; i < kTileCols * 8 / kBlock; ++i) {
+    const uint32_t id = tid + i * kBlock, r = id >> 3, q = id & 7;
+    if (tcol0 + r < cols && trow0 + q * 16 < rows) {
+      const u32x4 o = *reinterpret_cast<const u32x4*>(tile + r * kDualPitch + ((q ^ ((r >> 4) & 7u)) << 4));
+      st_stream(reinterpret_cast<u32x4*>(data + (uint64_t)(tcol0 + r) * rows + trow0 + q * 16), o);
+    }
+  }
+  // scales [cols/32, rows]: for each of the tile's row-direction blocks the bytes of its 128 rows
+  if (tid < kRowBlocks * 32) {
+    const uint32_t g = tid >> 5, r4 = (tid & 31) * 4, kb = tc * kRowBlocks + g;
+    if (kb < cols / 32 && trow0 + r4 < rows)
+      *reinterpret_cast<uint32_t*>(scale + (uint64_t)kb * rows + trow0 + r4) = *reinterpret_cast<const uint32_t*>(rtile + g * kDualRows + r4);
   }
 }
 

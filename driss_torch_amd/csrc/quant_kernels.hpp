@@ -56,10 +56,17 @@ __device__ __forceinline__ uint32_t absbits_of(const void* x, int64_t i) {
 template <int IN, int UNROLL, int NSCALES, bool NT>
 __global__ __launch_bounds__(kBlock) void amax_kernel(const void* __restrict__ x, Split sp,
                                                       uint8_t* __restrict__ ws, float* __restrict__ amax_out,
-                                                      float* __restrict__ scale_out, float fmax0, float fmax1) {
+                                                      float* __restrict__ scale_out, float fmax0, float fmax1,
+                                                      uint64_t* __restrict__ phase_log) {
   constexpr int kB = InTraits<IN>::kBytes, kV = InTraits<IN>::kVec;
   __shared__ uint32_t lds[kBlock / kWave];
   const int tid = threadIdx.x;
+  // phase_log (normally null): readings of the constant-rate 100 MHz counter per workgroup -- start,
+  // share loaded, workgroup's maximum known, atomics done -- for the benchmark's per-phase report
+  auto stamp = [&](int k) {
+    if (phase_log && tid == 0) phase_log[blockIdx.x * 4 + k] = wall_clock64();
+  };
+  stamp(0);
   const u32x4* v = reinterpret_cast<const u32x4*>(static_cast<const uint8_t*>(x) + sp.head * kB);
 
   uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
@@ -72,16 +79,39 @@ __global__ __launch_bounds__(kBlock) void amax_kernel(const void* __restrict__ x
       a2 = pk_absmax16(a2, w.z); a3 = pk_absmax16(a3, w.w);
     }
   };
-  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  // Batches of P loads, software-pipelined over two register sets: the loads of the next batch are
+  // issued before the current one is looked at, so P..2P loads per lane stay in flight and the memory
+  // system never runs dry between batches.  (Every load of the steady state is unconditional: the wait
+  // counts the compiler derives are exact only along straight-line code.)
+  constexpr int P = UNROLL / 2;
+  const int64_t stride = (int64_t)gridDim.x * kBlock, step = P * stride;
   int64_t i = (int64_t)blockIdx.x * kBlock + tid;
-  for (; i + (UNROLL - 1) * stride < sp.nvec; i += UNROLL * stride) {
-    u32x4 w[UNROLL];
+  auto whole_batch_at = [&](int64_t j) { return j + (P - 1) * stride < sp.nvec; };
+  auto load_batch = [&](u32x4 (&w)[P], int64_t j) {
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) w[u] = ld_maybe_stream<NT>(v + i + u * stride);
+    for (int u = 0; u < P; ++u) w[u] = ld_maybe_stream<NT>(v + j + u * stride);
+  };
+  auto absorb_batch = [&](const u32x4 (&w)[P]) {
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) absorb(w[u]);
+    for (int u = 0; u < P; ++u) absorb(w[u]);
+  };
+  if (whole_batch_at(i)) {
+    u32x4 wa[P], wb[P];
+    load_batch(wa, i);
+    i += step;
+    for (;;) {
+      if (!whole_batch_at(i)) { absorb_batch(wa); break; }
+      load_batch(wb, i);
+      i += step;
+      absorb_batch(wa);
+      if (!whole_batch_at(i)) { absorb_batch(wb); break; }
+      load_batch(wa, i);
+      i += step;
+      absorb_batch(wb);
+    }
   }
   for (; i < sp.nvec; i += stride) absorb(ld_maybe_stream<NT>(v + i));
+  stamp(1);
 
   uint32_t m;
   if constexpr (IN == DT_F32) {
@@ -95,6 +125,7 @@ __global__ __launch_bounds__(kBlock) void amax_kernel(const void* __restrict__ x
     if (tid < sp.tail) m = umax(m, absbits_of<IN>(x, sp.head + sp.nvec * kV + tid));
   }
   m = block_umax<kBlock / kWave>(m, lds);
+  stamp(2);
 
   // One relaxed device-scope atomic max per workgroup carries the partial; a second one on the
   // ticket tells the last workgroup to arrive.  No fence is needed: the max is an atomic with
@@ -128,6 +159,7 @@ __global__ __launch_bounds__(kBlock) void amax_kernel(const void* __restrict__ x
         }
       }
     }
+    stamp(3);
   }
 }
 
@@ -150,7 +182,8 @@ inline int launch_amax(const void* x, int64_t numel, void* ws, float* amax_out, 
   int grid = reduction_grid(sp.nvec, kUnroll, "amax.blocks_per_cu");
   uint8_t* w = static_cast<uint8_t*>(ws);
   const bool nt = nscales == 0 || tuning("amax.stream_before_cast");
-#define DT_AMAX(NS, NT) amax_kernel<IN, kUnroll, NS, NT><<<grid, kBlock, 0, stream>>>(x, sp, w, amax_out, scale_out, fmax0, fmax1)
+  uint64_t* const log = phase_log((size_t)grid * 32);
+#define DT_AMAX(NS, NT) amax_kernel<IN, kUnroll, NS, NT><<<grid, kBlock, 0, stream>>>(x, sp, w, amax_out, scale_out, fmax0, fmax1, log)
   if (nscales == 0) DT_AMAX(0, true);
   else if (nscales == 1) { if (nt) DT_AMAX(1, true); else DT_AMAX(1, false); }
   else { if (nt) DT_AMAX(2, true); else DT_AMAX(2, false); }
@@ -240,16 +273,34 @@ __global__ __launch_bounds__(kBlock) void cast_kernel(const void* __restrict__ x
   float s = scale[0], s2 = PAIR ? scale[1] : 0.f;
   if constexpr (ROUND_SCALE) { s = round_to_bf16(s); s2 = round_to_bf16(s2); }
   const u32x4* v = static_cast<const u32x4*>(x);
-  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  // batches of UNROLL loads, software-pipelined over two register sets (see amax_kernel)
+  constexpr int P = UNROLL;
+  const int64_t stride = (int64_t)gridDim.x * kBlock, step = P * stride;
   int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  for (; i + (UNROLL - 1) * stride < nvec; i += UNROLL * stride) {
-    u32x4 w[UNROLL];
+  auto whole_batch_at = [&](int64_t j) { return j + (P - 1) * stride < nvec; };
+  auto load_batch = [&](u32x4 (&w)[P], int64_t j) {
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) w[u] = ld_stream(v + i + u * stride);
+    for (int u = 0; u < P; ++u) w[u] = ld_stream(v + j + u * stride);
+  };
+  auto cast_batch = [&](const u32x4 (&w)[P], int64_t j) {
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      cast_vec<IN, OUT, ROUND_BF16>(w[u], s, out, i + u * stride);
-      if constexpr (PAIR) cast_vec<IN, OUT2, ROUND_BF16>(w[u], s2, out2, i + u * stride);
+    for (int u = 0; u < P; ++u) {
+      cast_vec<IN, OUT, ROUND_BF16>(w[u], s, out, j + u * stride);
+      if constexpr (PAIR) cast_vec<IN, OUT2, ROUND_BF16>(w[u], s2, out2, j + u * stride);
+    }
+  };
+  if (whole_batch_at(i)) {
+    u32x4 wa[P], wb[P];
+    load_batch(wa, i);
+    for (;;) {
+      if (!whole_batch_at(i + step)) { cast_batch(wa, i); i += step; break; }
+      load_batch(wb, i + step);
+      cast_batch(wa, i);
+      i += step;
+      if (!whole_batch_at(i + step)) { cast_batch(wb, i); i += step; break; }
+      load_batch(wa, i + step);
+      cast_batch(wb, i);
+      i += step;
     }
   }
   for (; i < nvec; i += stride) {
@@ -309,9 +360,9 @@ __global__ __launch_bounds__(kBlock) void cast_kernel_unaligned(const void* __re
 template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR>
 inline int launch_cast_impl(const void* x, int64_t numel, const float* scale, void* out, void* out2,
                             hipStream_t stream) {
-  // 4 loads in flight per lane and 2 workgroups per CU (32 KB per CU) is the best point of the
-  // measured grid {2, 4, 8 loads} x {1..32 workgroups}, alone and right behind the reduction
-  // (bf16 8192^2: 32.6 us against 33.8 with 8 x 2 and 41 with 8 x 8; more in flight is slower)
+  // Batches of 4 loads per lane, software-pipelined (4..8 in flight), from ONE workgroup per CU: the best
+  // point of the measured grid {1, 2, 4 workgroups per CU} (8192^2 bf16 32.5 / 32.9 / 36.0 us, fp32 54.2 /
+  // 60.1 / 66 us, bf16 to both fp8 types 45.1 / 45.3 / 47.8 us); more in flight is slower
   constexpr int kUnroll = 4;
   constexpr size_t kStoreAlign = IN == DT_F32 ? 4 : 8;
   uint8_t* o = static_cast<uint8_t*>(out);

@@ -21,6 +21,8 @@
 
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include <atomic>
 #include <mutex>
 
@@ -31,9 +33,26 @@ namespace dt {
 constexpr int kResRegVecs = 92;   // 16-byte vectors per lane kept in registers (368 VGPRs)
 constexpr int kResLdsVecs = 36;   // ... and in LDS (144 KiB per workgroup)
 constexpr int kResVecs = kResRegVecs + kResLdsVecs;
+constexpr int kResPipe = 4;       // loads per batch of the pipelined load phase (4..8 in flight per lane)
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<N, I + 1>(f);
+  }
+}
 constexpr size_t kResLdsBytes = (size_t)kResLdsVecs * kBlock * 16;
 constexpr size_t kWsDepart = 192;  // u32 departure counter of the grid barrier, zero between launches
-constexpr size_t kWsRelease = 256; // u64 release word of the grid barrier (a cache line of its own), zero between launches
+// u64 release words of the grid barrier, zero between launches: kWsReleaseWords of them, kWsReleaseStep
+// bytes apart.  A workgroup polls word (workgroup index % kWsReleaseWords).  One word polled by every
+// workgroup is one memory location serving a few hundred requests per polling round, one after the other:
+// the release then reaches the workgroups spread over 3 us (measured with the phase log).
+constexpr size_t kWsRelease = 1024;
+constexpr size_t kWsReleaseStep = 256;
+constexpr uint32_t kWsReleaseWords = 8;
+static_assert(kWsRelease + kWsReleaseWords * kWsReleaseStep <= kWsBytes, "release words fit the workspace");
 constexpr size_t kWsTimeout = 196; // u32, set (and left set) if a barrier wait ever gave up
 
 // One vector to e4m3fn and e5m2 at once, for products that cannot be NaN.  The two scales are
@@ -111,6 +130,7 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
   };
   constexpr int kResBatch = 16;
   static_assert(kResRegVecs % 4 == 0 && kResLdsVecs % 4 == 0, "batches");
+  static_assert(kResLdsVecs % kResPipe == 0, "a pipelined batch is LDS slots or register slots, not both");
   // Vector slots k >= nk lie past the end for every lane of this workgroup: a tensor smaller than
   // the chip's capacity skips whole batches (a branch the workgroup takes as one), in both passes.
   const uint32_t block_first = blockIdx.x * kBlock;
@@ -126,35 +146,76 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
       __builtin_amdgcn_sched_barrier(0);
     }
   }
-  // the LDS part first (through a batch of registers), then the register part in place
+  // The kept part: LDS slots first (through temporaries), then the register slots in place.
+  if (nk > (uint32_t)(kResVecs - 2 * kResBatch)) {
+    // A (nearly) full share: one unconditional stream of batches of kResPipe loads, the loads of batch
+    // n + 1 issued before batch n is looked at, so that the memory system never runs dry between
+    // batches (load phase of 8192 x 8192 bf16: 21.8 -> see bench).  No branch anywhere: a slot past the
+    // end reads the last vector again and counts as zeros.
+    constexpr int kSeq = kResVecs, kBatches = (kSeq + kResPipe - 1) / kResPipe;
+    u32x4 t[2][kResPipe];  // temporaries of the LDS slots (position p < kResLdsVecs of the sequence)
+    auto issue = [&](auto n_tag) {
+      constexpr int n = decltype(n_tag)::value;
 #pragma unroll
-  for (int b = 0; b < kResLdsVecs; b += kResBatch) {
-    if ((uint32_t)(kResRegVecs + b) >= nk) break;
-    u32x4 t[kResBatch];
-#pragma unroll
-    for (int j = 0; j < kResBatch; ++j)
-      if (b + j < kResLdsVecs) t[j] = fetch(kResRegVecs + b + j);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int j = 0; j < kResBatch; ++j)
-      if (b + j < kResLdsVecs) {
-        absorb(kResRegVecs + b + j, t[j]);
-        keep[(b + j) * kBlock + tid] = t[j];
+      for (int j = 0; j < kResPipe; ++j) {
+        const int p = n * kResPipe + j;
+        if (p >= kSeq) continue;
+        if (p < kResLdsVecs) t[n & 1][j] = fetch(kResRegVecs + p);
+        else r[p - kResLdsVecs] = fetch(p - kResLdsVecs);
       }
-    __builtin_amdgcn_sched_barrier(0);
-  }
+    };
+    auto retire = [&](auto n_tag) {
+      constexpr int n = decltype(n_tag)::value;
 #pragma unroll
-  for (int b = 0; b < kResRegVecs; b += kResBatch) {
-    if ((uint32_t)b >= nk) break;
+      for (int j = 0; j < kResPipe; ++j) {
+        const int p = n * kResPipe + j;
+        if (p >= kSeq) continue;
+        if (p < kResLdsVecs) {
+          absorb(kResRegVecs + p, t[n & 1][j]);
+          keep[p * kBlock + tid] = t[n & 1][j];
+        } else {
+          absorb(p - kResLdsVecs, r[p - kResLdsVecs]);
+        }
+      }
+    };
+    issue(std::integral_constant<int, 0>{});
+    static_for<kBatches>([&](auto n_tag) {
+      constexpr int n = decltype(n_tag)::value;
+      if constexpr (n + 1 < kBatches) issue(std::integral_constant<int, n + 1>{});
+      __builtin_amdgcn_sched_barrier(0);
+      retire(n_tag);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  } else {
 #pragma unroll
-    for (int j = 0; j < kResBatch; ++j)
-      if (b + j < kResRegVecs) r[b + j] = fetch(b + j);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int j = 0; j < kResBatch; ++j)
-      if (b + j < kResRegVecs) absorb(b + j, r[b + j]);
-    __builtin_amdgcn_sched_barrier(0);
-  }
+    for (int b = 0; b < kResLdsVecs; b += kResBatch) {
+      if ((uint32_t)(kResRegVecs + b) >= nk) break;
+      u32x4 t[kResBatch];
+  #pragma unroll
+      for (int j = 0; j < kResBatch; ++j)
+        if (b + j < kResLdsVecs) t[j] = fetch(kResRegVecs + b + j);
+      __builtin_amdgcn_sched_barrier(0);
+  #pragma unroll
+      for (int j = 0; j < kResBatch; ++j)
+        if (b + j < kResLdsVecs) {
+          absorb(kResRegVecs + b + j, t[j]);
+          keep[(b + j) * kBlock + tid] = t[j];
+        }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  #pragma unroll
+    for (int b = 0; b < kResRegVecs; b += kResBatch) {
+      if ((uint32_t)b >= nk) break;
+  #pragma unroll
+      for (int j = 0; j < kResBatch; ++j)
+        if (b + j < kResRegVecs) r[b + j] = fetch(b + j);
+      __builtin_amdgcn_sched_barrier(0);
+  #pragma unroll
+      for (int j = 0; j < kResBatch; ++j)
+        if (b + j < kResRegVecs) absorb(b + j, r[b + j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+}
   uint32_t m;
   if constexpr (IN == DT_F32) {
     m = umax(umax(a0, a1), umax(a2, a3));
@@ -167,27 +228,28 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
   stamp(1);
 
   // ---- grid barrier on the reduction's atomics: fold the partial into the running maximum,
-  // take a ticket, wait until every workgroup has taken one, read the maximum.  The last
-  // workgroup to leave publishes amax and the scales and re-arms the workspace.
+  // take a ticket, wait until every workgroup has taken one, read the maximum.
   // The waiting workgroups poll a word of its own (another cache line): polling the line the
   // arrivals update slows those atomics down for everybody (measured: 8 us -> see bench).
   uint32_t* running = reinterpret_cast<uint32_t*>(ws + kWsRunning);
   uint32_t* ticket = reinterpret_cast<uint32_t*>(ws + kWsTicket);
   uint32_t* depart = reinterpret_cast<uint32_t*>(ws + kWsDepart);
-  uint64_t* release = reinterpret_cast<uint64_t*>(ws + kWsRelease);  // (1 << 32) | amax bits once everybody has arrived
+  // (1 << 32) | amax bits once everybody has arrived; this workgroup polls its own copy
+  uint64_t* release = reinterpret_cast<uint64_t*>(ws + kWsRelease + (blockIdx.x % kWsReleaseWords) * kWsReleaseStep);
   if (tid == 0) {
     uint32_t before = __hip_atomic_fetch_max(running, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     uint32_t one = 1u;  // the ticket depends on the returned value, so the two atomics stay ordered
     asm volatile("v_and_or_b32 %0, %1, 0, %0" : "+v"(one) : "v"(before));
     const uint32_t t = __hip_atomic_fetch_add(ticket, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    uint32_t bits, released = 0u;
+    uint32_t bits;
     if (t == gridDim.x - 1) {
       // last to arrive: every other workgroup's maximum was folded in before it took its ticket
       bits = __hip_atomic_load(running, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      // an exchange, not a store: its returned value (always 0) is folded into the departure below, so
-      // this workgroup cannot be counted as departed -- and the release word cannot be re-armed by the
-      // last one to leave -- before the release has been performed
-      released = (uint32_t)__hip_atomic_exchange(release, (1ull << 32) | bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const uint64_t word = (1ull << 32) | bits;
+#pragma unroll
+      for (uint32_t j = 0; j < kWsReleaseWords; ++j)
+        __hip_atomic_store(reinterpret_cast<uint64_t*>(ws + kWsRelease + j * kWsReleaseStep), word, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
     } else {
       uint32_t spins = 0;
       uint64_t rel;
@@ -204,27 +266,6 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
       bits = (uint32_t)rel;
     }
     bcast = bits;
-    uint32_t dep = 1u;
-    asm volatile("v_and_or_b32 %0, %1, 0, %0" : "+v"(dep) : "v"(bits));  // leave only after the read
-    asm volatile("v_and_or_b32 %0, %1, 0, %0" : "+v"(dep) : "v"(released));  // ... and after the release
-    if (__hip_atomic_fetch_add(depart, dep, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1) {
-      __hip_atomic_store(running, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(depart, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(release, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const float amax = as_f32(bits);
-      float* wscale = reinterpret_cast<float*>(ws + kWsScale);
-      *reinterpret_cast<float*>(ws + kWsAmax) = amax;
-      if (amax_out) *amax_out = amax;
-      const float s0 = amax_to_scale(amax, fmax0);
-      wscale[0] = s0;
-      if (scale_out) scale_out[0] = s0;
-      if constexpr (PAIR) {
-        const float s1 = amax_to_scale(amax, fmax1);
-        wscale[1] = s1;
-        if (scale_out) scale_out[1] = s1;
-      }
-    }
   }
   __syncthreads();
   stamp(2);
@@ -299,6 +340,35 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
     __syncthreads();
     stamp(3);
   }
+  // ---- departure, at the very end: counted here and not at the barrier, where the atomic's round trip
+  // (the 256 of them queue on one address) held every workgroup back by 1.5-3 us before its stores.  The
+  // last workgroup to leave publishes amax and the scales and re-arms the workspace for the next launch.
+  if (tid == 0) {
+    // everything this wave has sent to memory has been performed, the release words of the last
+    // arriver included: whoever finds itself last may put them back to zero
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (__hip_atomic_fetch_add(depart, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1) {
+      __hip_atomic_store(running, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(depart, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (uint32_t j = 0; j < kWsReleaseWords; ++j)
+        __hip_atomic_store(reinterpret_cast<uint64_t*>(ws + kWsRelease + j * kWsReleaseStep), 0ull, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      const float amax_final = as_f32(bcast);
+      float* wscale = reinterpret_cast<float*>(ws + kWsScale);
+      *reinterpret_cast<float*>(ws + kWsAmax) = amax_final;
+      if (amax_out) *amax_out = amax_final;
+      const float s0 = amax_to_scale(amax_final, fmax0);
+      wscale[0] = s0;
+      if (scale_out) scale_out[0] = s0;
+      if constexpr (PAIR) {
+        const float s1 = amax_to_scale(amax_final, fmax1);
+        wscale[1] = s1;
+        if (scale_out) scale_out[1] = s1;
+      }
+    }
+  }
 }
 
 // Host-side chaining of resident launches (see launch_resident_impl).
@@ -313,9 +383,6 @@ struct ResidentGate {
   // next per-tensor dynamic quantization on that device.
   volatile uint32_t* gave_up_host[kMaxDevices] = {};
   uint32_t* gave_up_dev[kMaxDevices] = {};
-  // device buffer for the per-phase clock readings of the next resident launches (benchmarking), or null
-  std::atomic<uint64_t*> phase_log{nullptr};
-  std::atomic<size_t> phase_log_bytes{0};
 };
 inline ResidentGate& resident_gate() {
   static ResidentGate* g = new ResidentGate();  // leaked on purpose: no HIP calls at process exit
@@ -429,8 +496,7 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
     gate.gave_up_host[dev] = static_cast<volatile uint32_t*>(host);
     gate.gave_up_dev[dev] = static_cast<uint32_t*>(devp);
   }
-  uint64_t* phase_log = gate.phase_log.load(std::memory_order_relaxed);
-  if (phase_log && gate.phase_log_bytes.load(std::memory_order_relaxed) < (size_t)grid * 32) phase_log = nullptr;
+  uint64_t* const log = phase_log((size_t)grid * 32);
   if (gate.used[dev] && gate.last_stream[dev] != stream) {
     // mark the tail of the stream that ran the previous resident kernel and wait for it here
     if (!gate.event[dev] && hipEventCreateWithFlags(&gate.event[dev], hipEventDisableTiming) != hipSuccess) {
@@ -447,7 +513,7 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
     }
   }
   kernel<<<(unsigned)grid, kBlock, kResLdsBytes, stream>>>(x, nvec, tail, w, o, o2, amax_out, scale_out, fmax0, fmax1,
-                                                         spin_limit, gate.gave_up_dev[dev], phase_log);
+                                                         spin_limit, gate.gave_up_dev[dev], log);
   const int st = launch_status();
   if (st == DT_OK) {
     gate.used[dev] = true;

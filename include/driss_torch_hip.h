@@ -182,10 +182,11 @@ DT_API int dt_dynamic_scaled_quant_rowwise(const void* x, int in_dtype, int64_t 
  * scale_layout DT_SCALE_BLOCKED writes the scale matrix directly in the layout
  * dt_mx_fp8_bf16 reads (dt_blocked_scale_bytes(scale_rows, scale_cols) bytes, padding
  * zeroed); it needs the scale matrix to be [outer, inner/32], i.e. (axis 1, transpose 0)
- * or (axis 0, transpose 1).  in_dtype F32, BF16 or F16.  x aligned to its element: the fast
- * kernels want 16 bytes; an x off a 16-byte boundary keeps its vector loads for (axis 1,
- * transpose 0) and takes a much slower general kernel for the other orientations, as does
- * (axis 1, transpose 1) always.                                                            */
+ * or (axis 0, transpose 1).  in_dtype F32, BF16 or F16.  x only has to be aligned to its element (a
+ * view that starts anywhere in its buffer keeps the 16-byte loads).  Shapes and output alignments the
+ * tiled kernels do not take run on a much slower general kernel: data not 16-byte aligned (axis 1,
+ * transpose 0: 8-byte), scale not 4-byte aligned (axis 0, transpose 0: 8-byte), cols not a multiple of
+ * 4 for axis 0, rows not a multiple of 16 for (axis 1, transpose 1).                          */
 DT_API int dt_mx_fp8_quantize(const void* x, int in_dtype, int64_t rows, int64_t cols, int axis,
                               int transpose, int out_dtype, int scale_layout, void* data,
                               uint8_t* scale, dt_stream_t stream);
@@ -273,9 +274,10 @@ DT_API int dt_set_tuning(const char* key, int value);
 DT_API int dt_get_tuning(const char* key, int* value);
 
 /* Benchmarking aid, no counterpart in the reference: while a device buffer is set here (8-byte aligned,
- * at least 32 bytes per CU; NULL switches it off), every one-kernel dynamic quantization writes four
- * readings of the 100 MHz constant-rate counter per workgroup into it (uint64[workgroup][4]: start,
- * share loaded and reduced, released from the grid barrier, stores done).                          */
+ * at least 32 bytes per workgroup of the kernel's grid; NULL switches it off), every one-kernel dynamic
+ * quantization and every amax reduction writes four readings of the 100 MHz constant-rate counter
+ * per workgroup into it (uint64[workgroup][4]: start; share loaded and reduced / loaded; released from
+ * the grid barrier / workgroup maximum known; stores done / atomics done).                          */
 DT_API int dt_set_phase_log(void* device_buffer, size_t bytes);
 
 #ifdef __cplusplus

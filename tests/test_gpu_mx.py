@@ -79,9 +79,8 @@ def test_mx_cast_special_blocks(d, in_dtype, axis, transpose):
 
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32, torch.float16])
 def test_mx_cast_input_off_a_16_byte_boundary(d, in_dtype):
-    """a contiguous view that starts one element into its buffer: the row-wise cast keeps its 16-byte
-    loads (element-aligned vector type), the other orientations go through the generic kernel; all
-    of them against the oracle"""
+    """a contiguous view that starts one element into its buffer: every orientation keeps its tiled
+    kernel (the loads go through element-aligned vector types); all of them against the oracle"""
     rows, cols = 96, 544
     a = util.student_t((rows, cols), 61, in_dtype)
     buf = torch.empty(a.numel() + 3, dtype=in_dtype, device="cuda")
@@ -96,9 +95,32 @@ def test_mx_cast_input_off_a_16_byte_boundary(d, in_dtype):
     cd, cs = co.mx_quantize(a, 0, True)
     data, scale = d.mx_fp8_quantize(x, 32, 0, True)
     assert torch.equal(util.codes(data), cd) and torch.equal(util.codes(scale), cs.flatten())
-    dr, sr, dc, sc = d.mx_fp8_quantize_dual(x)   # falls back to the two single casts
+    dr, sr, dc, sc = d.mx_fp8_quantize_dual(x)
     assert torch.equal(util.codes(dr), rd) and torch.equal(util.codes(sr), rs.flatten())
     assert torch.equal(util.codes(dc), cd) and torch.equal(util.codes(sc), cs.flatten())
+    for axis, transpose in ((0, False), (1, True)):
+        wd, ws = co.mx_quantize(a, axis, transpose)
+        data, scale = d.mx_fp8_quantize(x, 32, axis, transpose)
+        assert torch.equal(util.codes(data), wd) and torch.equal(util.codes(scale), ws.flatten())
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(16, 32), (48, 96), (272, 544), (128, 8192), (4112, 256)], ids=lambda s: f"{s[0]}x{s[1]}")
+def test_mx_cast_rows_with_transposed_payload(d, in_dtype, shape):
+    """(axis 1, transpose): the row-wise cast written as [cols, rows] with scales [cols/32, rows]; equal to the
+    row-wise cast transposed, NaN and zero blocks included, on row counts that are multiples of 16 but not
+    of 32 or 128, and through the general kernel when they are not multiples of 16"""
+    a = util.student_t(shape, 901 + shape[0], in_dtype)
+    a[0, :32] = 0
+    a[shape[0] - 1, 5] = float("nan")
+    rd, rs = co.mx_quantize(a, 1, False)
+    data, scale = d.mx_fp8_quantize(a.cuda(), 32, 1, True)
+    assert data.shape == (shape[1], shape[0])
+    assert torch.equal(util.codes(data), rd.t()) and torch.equal(util.codes(scale).view(shape[1] // 32, shape[0]), rs.t())
+    odd = a[:shape[0] - 3].contiguous() if shape[0] > 3 else a
+    rd, rs = co.mx_quantize(odd, 1, False)
+    data, scale = d.mx_fp8_quantize(odd.cuda(), 32, 1, True)
+    assert torch.equal(util.codes(data), rd.t()) and torch.equal(util.codes(scale).view(shape[1] // 32, -1), rs.t())
 
 
 def test_mx_cast_blocked_scales_and_errors(d, cabi):
