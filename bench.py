@@ -77,6 +77,59 @@ def time_launches(fn, nsets, steps, warmup):
     return start.elapsed_time(end) * 1e3 / steps
 
 
+_NOT_LAUNCHES = {"dt_workspace_bytes", "dt_blocked_scale_bytes", "dt_mx_gemm_workspace_bytes", "dt_status_string",
+                 "dt_get_tuning", "dt_set_tuning", "dt_workspace_init", "dt_mx_gemm_workspace_init", "dt_abi_version",
+                 "dt_set_phase_log", "dt_dynamic_quant_gave_up"}
+
+
+class _Recorder:
+    """Stands in for the C-ABI library handle while one call of a wrapper is noted down."""
+
+    def __init__(self, lib):
+        self._lib, self.calls = lib, []
+
+    def __getattr__(self, name):
+        fn = getattr(self._lib, name)
+        if name in _NOT_LAUNCHES or not name.startswith("dt_"):
+            return fn
+
+        def noted(*args):
+            self.calls.append((fn, args))
+            return fn(*args)
+
+        return noted
+
+
+def bind(cabi, run, *args):
+    """run(*args) once, noting the C-ABI entry points it reaches with their plain arguments (pointers,
+    sizes, stream); returns a callable that repeats exactly those calls.  The Python wrappers in cabi.py
+    cost 10-20 us per call (tensor attribute look-ups), more than some kernels take: the timed loops call
+    the C ABI the way a compiled host would."""
+    rec, saved = _Recorder(cabi.lib()), cabi._lib
+    cabi._lib = rec
+    try:
+        run(*args)
+    finally:
+        cabi._lib = saved
+    calls = rec.calls
+    assert calls, "the wrapper made no C-ABI call"
+    if len(calls) == 1:
+        fn, a = calls[0]
+
+        def replay_one():
+            if fn(*a):
+                raise RuntimeError("C-ABI call failed in the timed loop")
+
+        return replay_one
+
+    def replay():
+        for f, a_ in calls:
+            if f(*a_):
+                raise RuntimeError("C-ABI call failed in the timed loop")
+
+    return replay
+
+
 def nsets_for(bytes_per_set):
     """buffer sets needed so a set is evicted from the memory-side cache before it is reused"""
     return max(2, -(-2 * MALL_BYTES // bytes_per_set) + 1)
@@ -110,7 +163,9 @@ def main():
     torch.cuda.set_device(dev)
     K, W = args.steps, args.warmup
     if args.gemm_only:
-        print(json.dumps({"kernels": extra_kernels(torch, cabi, dev, K, W, gemm_only=True)}))
+        ph = {} if args.phases else None
+        rows = extra_kernels(torch, cabi, dev, K, W, gemm_only=True, phases=ph)
+        print(json.dumps({"kernels": rows, "phases": ph} if ph else {"kernels": rows}))
         return
 
     # ------------------------------------------------------------ headline step: config 2
@@ -133,16 +188,19 @@ def main():
     scale_out = torch.empty(2, dtype=torch.float32, device=dev)
     mode = cabi.ROUND_BF16_SCALE_PRODUCT
 
+    steps_bound = [bind(cabi, lambda s=s: cabi.dynamic_scaled_quant_pair(xs[s], mode, o4[s], o5[s], amax_out, scale_out))
+                   for s in range(ns)]
+    amax_bound = [bind(cabi, lambda s=s: cabi.amax_scales(xs[s], amax_out, scale_out)) for s in range(ns)]
+    cast_bound = [bind(cabi, lambda s=s: cabi.saturated_cast_pair(xs[s], scale_out, mode, o4[s], o5[s])) for s in range(ns)]
+
     def step(i):
-        s = i % ns
-        cabi.dynamic_scaled_quant_pair(xs[s], mode, o4[s], o5[s], amax_out, scale_out)
+        steps_bound[i % ns]()
 
     def step_staged(i, ev):
         # the same two kernels through the staged entry points, with events around the second
-        s = i % ns
-        cabi.amax_scales(xs[s], amax_out, scale_out)
+        amax_bound[i % ns]()
         ev[0].record()
-        cabi.saturated_cast_pair(xs[s], scale_out, mode, o4[s], o5[s])
+        cast_bound[i % ns]()
         ev[1].record()
 
     # timed region 1: K whole steps, nothing between the launches -> `value`
@@ -159,7 +217,7 @@ def main():
 
     # timed region 2: the step is one kernel (the tensor fits the chip, see resident_kernels.hpp):
     # K launches between one pair of HIP events on the launch stream -> `roofline`
-    step_us = time_launches(step, ns, K, 0)
+    step_us = time_launches(step, ns, K, W)
     step_gbs = step_bytes / (step_us * 1e-6) / 1e9
 
     phases = None
@@ -169,6 +227,7 @@ def main():
         amax_tmp = torch.empty(1, dtype=torch.float32, device=dev)
         phases["amax_kernel, bf16 [8192,8192]"] = kernel_phases(
             torch, cabi, lambda i: cabi.amax(xs[i % ns], amax_tmp), ["load", "workgroup reduce", "atomics"])
+        del amax_tmp
 
     # for comparison: the two-kernel path every larger tensor takes (amax, then cast), the cast
     # bracketed by an event pair per launch (adds about 4 us of dispatch latency to it)
@@ -220,8 +279,6 @@ def main():
                             "cast_kernel(pair) GBs (4 B per element)": round(cast_bytes / (cast_us * 1e-6) / 1e9, 1),
                             "cast_kernel(pair) traffic": cast_traffic},
     }
-    if phases:
-        result["phases"] = phases
     if args.calibrate_copy:
         src = xs[0]
         dst = torch.empty_like(src)
@@ -233,7 +290,9 @@ def main():
     torch.cuda.empty_cache()
 
     if not args.no_extra:
-        result["kernels"] = extra_kernels(torch, cabi, dev, K, W)
+        result["kernels"] = extra_kernels(torch, cabi, dev, K, W, phases=phases)
+    if phases:
+        result["phases"] = phases
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, x_cpu, step_bytes)
     print(json.dumps(result))
@@ -285,7 +344,63 @@ def kernel_phases(torch, cabi, launch, names, launches=20):
     return out
 
 
-def extra_kernels(torch, cabi, dev, K, W, gemm_only=False):
+def gemm_timeline(torch, cabi, launch, launches=5):
+    """Where the block-scaled GEMM spends its time: with a phase log set every workgroup (= output tile)
+    writes four readings of the 100 MHz constant-rate counter (start, K loop entered, K loop left, output
+    stored) and the XCD and CU it ran on.  Medians over `launches` launches, each in a train of warm
+    launches (the clocks need tens of launches to settle); microseconds."""
+    import collections
+
+    L = cabi.lib()
+    log = torch.zeros((8192, 8), dtype=torch.int64, device="cuda")
+    rows = []
+    for _ in range(launches):
+        for _ in range(30):
+            launch()
+        assert L.dt_set_phase_log(log.data_ptr(), log.numel() * 8) == 0
+        try:
+            log.zero_()
+            launch()
+            torch.cuda.synchronize()
+        finally:
+            L.dt_set_phase_log(None, 0)
+        d = log.cpu()
+        d = d[d[:, 0] > 0]
+        if d.numel() == 0:
+            return None
+        t = (d[:, :4] - d[:, 0].min()).double() / 100.0
+        xcc = (d[:, 4] & 0xF).tolist()
+        hw = d[:, 5].tolist()
+        per_cu = collections.defaultdict(list)
+        for i in range(t.shape[0]):
+            per_cu[(xcc[i], (hw[i] >> 8) & 0xF, (hw[i] >> 12) & 1, (hw[i] >> 13) & 7)].append(t[i].tolist())
+        gaps = []
+        for v in per_cu.values():
+            v.sort()
+            gaps += [b[0] - a[3] for a, b in zip(v, v[1:])]
+        med = lambda v: float(torch.as_tensor(v, dtype=torch.float64).median())  # noqa: E731
+        loop = t[:, 2] - t[:, 1]
+        by_xcd = lambda col: [round(med([col[i] for i in range(len(xcc)) if xcc[i] == x]), 2) for x in sorted(set(xcc))]  # noqa: E731
+        rows.append({
+            "tiles": int(t.shape[0]), "CUs": len(per_cu), "kernel span (first start to last store)": float(t[:, 3].max()),
+            "per tile: prologue (first stages and fragments in)": med(t[:, 1] - t[:, 0]),
+            "per tile: K loop": med(loop), "per tile: epilogue (convert, stage, stores issued and performed)": med(t[:, 3] - t[:, 2]),
+            "per CU: gap between a tile's end and the next one's start": med(gaps) if gaps else 0.0,
+            "K loop by XCD": by_xcd(loop.tolist()),
+            "last store by XCD": [round(max(t[i, 3].item() for i in range(len(xcc)) if xcc[i] == x), 2) for x in sorted(set(xcc))],
+        })
+    out = {}
+    for k in rows[0]:
+        if isinstance(rows[0][k], list):
+            out[k] = [round(statistics.median(r[k][x] for r in rows), 2) for x in range(len(rows[0][k]))]
+        else:
+            out[k] = round(statistics.median(r[k] for r in rows), 2)
+    out["launches"] = len(rows)
+    out["unit"] = "us (100 MHz counter)"
+    return out
+
+
+def extra_kernels(torch, cabi, dev, K, W, gemm_only=False, phases=None):
     """Every other kernel of the path at its benchmark config: rotated (HBM) and hot-cache."""
     rows = []
 
@@ -294,8 +409,9 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False):
         set_bytes = sum(t.numel() * t.element_size() for t in one if isinstance(t, torch.Tensor))
         ns = nsets_for(set_bytes)
         sets = [one] + [make_set(i) for i in range(1, ns)]
-        us = time_launches(lambda i: run(*sets[i]), ns, K, W)
-        us_hot = time_launches(lambda i: run(*sets[0]), 1, K, W)
+        bound = [bind(cabi, run, *st) for st in sets]
+        us = time_launches(lambda i: bound[i](), ns, K, W)
+        us_hot = time_launches(lambda i: bound[0](), 1, K, W)
         gbs = nbytes / (us * 1e-6) / 1e9
         rows.append({"kernel": name, "workload": workload, "bound": "hbm", "avg_us": round(us, 2),
                      "achieved_GBs": round(gbs, 1), "frac_of_8TBs": round(gbs / HBM_PEAK_GBS, 4),
@@ -389,19 +505,35 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False):
     out = torch.empty((M, N), dtype=bf16, device=dev)
     del a, b
     # the clocks take tens of milliseconds of sustained MFMA load to settle: warm up for ~30 launches
-    us = time_launches(lambda i: cabi.mx_fp8_bf16(a_data, b_data, sfa, sfb, out), 1, max(20, K // 2), max(30, W))
+    gemm8 = bind(cabi, lambda: cabi.mx_fp8_bf16(a_data, b_data, sfa, sfb, out))
+    us = time_launches(lambda i: gemm8(), 1, max(20, K // 2), max(30, W))
     flops = 2.0 * M * N * Kd
     tf = flops / (us * 1e-6) / 1e12
+    if phases is not None:
+        phases["mx_gemm_kernel, config 5 (8192^3 e4m3)"] = gemm_timeline(
+            torch, cabi, gemm8)
     rows.append({"kernel": "mx_fp8_bf16", "workload": "config 5: 8192^3 e4m3 x e4m3, E8M0 block-32 scales -> bf16",
                  "bound": "mfma", "avg_us": round(us, 2), "achieved_TFLOPs": round(tf, 1),
                  "frac_of_fp8_peak": round(tf / FP8_PEAK_TFLOPS, 4), "flops": flops})
+    # The same launch on operands of ones (payload 0x38, scale bytes 127): the same schedule and the same
+    # data movement with almost no switching in the multipliers.  The difference to the row above is the
+    # shader clock the power management allows (cycles per launch are the same, see profiles/).
+    ones_a = torch.full((M, Kd), 0x38, dtype=torch.uint8, device=dev).view(e4)
+    ones_s = torch.full_like(sfa, 127)
+    gemm1 = bind(cabi, lambda: cabi.mx_fp8_bf16(ones_a, ones_a, ones_s, ones_s, out))
+    us1 = time_launches(lambda i: gemm1(), 1, max(20, K // 2), max(30, W))
+    rows.append({"kernel": "mx_fp8_bf16", "workload": "8192^3, every operand element 1.0 (same schedule and traffic, little switching power)",
+                 "bound": "mfma", "avg_us": round(us1, 2), "achieved_TFLOPs": round(flops / (us1 * 1e-6) / 1e12, 1),
+                 "frac_of_fp8_peak": round(flops / (us1 * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4), "flops": flops})
+    del ones_a, ones_s
     # two shapes off the 8192^3 grid, on row slices of the same operands (blocked scales are
     # stored by 128-row chunks, so a row prefix of the operand owns a prefix of its scales)
     for m_rows, n_rows, what in ((16, 8192, "16 rows: K shared between 4 workgroups per 128x128 tile"),
                                  (1024, 8192, "128 tiles of 256x256 on 256 CUs: runs as 256 tiles of 256x128")):
         sa_rows, sb_rows = -(-m_rows // 128) * 128 * (Kd // 32), -(-n_rows // 128) * 128 * (Kd // 32)
         ops = (a_data[:m_rows], b_data[:n_rows], sfa[:sa_rows], sfb[:sb_rows], out[:m_rows, :n_rows])
-        us = time_launches(lambda i: cabi.mx_fp8_bf16(*ops), 1, max(20, K // 2), 10)
+        gemm_small = bind(cabi, lambda: cabi.mx_fp8_bf16(*ops))
+        us = time_launches(lambda i: gemm_small(), 1, max(20, K // 2), 10)
         fl = 2.0 * m_rows * n_rows * Kd
         rows.append({"kernel": "mx_fp8_bf16", "workload": f"{m_rows}x{n_rows}x{Kd} e4m3 ({what})", "bound": "mfma",
                      "avg_us": round(us, 2), "achieved_TFLOPs": round(fl / (us * 1e-6) / 1e12, 1), "flops": fl})
@@ -409,7 +541,8 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False):
     del a_data, b_data
     a4, s4a = cabi.mx_fp4_quantize(rnd((M, Kd), bf16, 1), cabi.SCALE_BLOCKED)
     b4, s4b = cabi.mx_fp4_quantize(rnd((N, Kd), bf16, 2), cabi.SCALE_BLOCKED)
-    us = time_launches(lambda i: cabi.mx_fp4_bf16(a4, b4, s4a, s4b, out), 1, max(20, K // 2), max(30, W))
+    gemm4 = bind(cabi, lambda: cabi.mx_fp4_bf16(a4, b4, s4a, s4b, out))
+    us = time_launches(lambda i: gemm4(), 1, max(20, K // 2), max(30, W))
     tf = flops / (us * 1e-6) / 1e12
     rows.append({"kernel": "mx_fp4_bf16", "workload": "8192^3 e2m1 x e2m1, E8M0 block-32 scales -> bf16",
                  "bound": "mfma", "avg_us": round(us, 2), "achieved_TFLOPs": round(tf, 1),

@@ -70,8 +70,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const uint8_t* __restrict__ sfa,
     const uint8_t* __restrict__ sfb, int M, int N, int K, int64_t lda, int64_t ldb, uint16_t* __restrict__ out,
     int64_t ldo, int tiles_m, int tiles_n, int wide_stores, int splits, v4f* __restrict__ partial,
-    uint32_t* __restrict__ tickets, int first_block) {
+    uint32_t* __restrict__ tickets, int first_block, uint64_t* __restrict__ phase_log) {
   constexpr bool SPLIT = MODE == kSplitK;
+  // phase_log (normally null; dt_set_phase_log): per workgroup four readings of the 100 MHz constant-rate
+  // counter -- start, K loop entered, K loop left, output stored -- and where it ran (XCC_ID, HW_ID).
+  // The readings are taken always (three scalar reads per tile) and stored at the very end.
+  const uint64_t t_start = wall_clock64();
   static_assert(!(SPLIT && TOUCH), "the prefetch shares assume that a workgroup walks the whole K");
   static_assert(MODE != kQuads || (BM == 128 && BN == 128), "quadrants of a 256 x 256 tile");
   static_assert(MODE != kHalves || (BM == 256 && BN == 128), "halves of a 256 x 256 tile");
@@ -350,6 +354,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     }
   }
 
+  const uint64_t t_loop = wall_clock64();
   int slot = 0;  // ring slot of step ks
   int ks = 0;
   do {  // k_steps >= 1
@@ -462,6 +467,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // (the no-ops cover the distance an assembly-written MFMA needs before its result is read)
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
+  const uint64_t t_loop_end = wall_clock64();
 
   if constexpr (SPLIT) {
     __shared__ uint32_t drawn;
@@ -559,6 +565,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
       *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(src + r * kEpiPitch);
       dst += pass_stride;
     }
+    if (phase_log) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (threadIdx.x == 0) {
+        uint64_t* const e = phase_log + (size_t)blockIdx.x * 8;
+        e[0] = t_start; e[1] = t_loop; e[2] = t_loop_end; e[3] = wall_clock64();
+        e[4] = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11));  // XCC_ID
+        e[5] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_ID
+      }
+    }
     return;
   }
 #pragma unroll
@@ -615,7 +630,7 @@ int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const ui
   kernel<<<(unsigned)grid, WAVES_M * WAVES_N * kWave, lds_bytes, stream>>>(
       a, b, sfa, sfb, (int)M, (int)N, (int)K, lda, ldb, static_cast<uint16_t*>(out), ldo, tiles_m, tiles_n,
       (ldo % 8 == 0 && aligned(out, 16)) ? 1 : 0, splits, ws ? reinterpret_cast<v4f*>(ws + kSplitTicketBytes) : nullptr,
-      reinterpret_cast<uint32_t*>(ws), first_block);
+      reinterpret_cast<uint32_t*>(ws), first_block, phase_log((size_t)grid * 64));
   return launch_status();
 }
 
