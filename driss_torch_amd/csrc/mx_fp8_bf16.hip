@@ -129,13 +129,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   if constexpr (PARTS) {
     if (m0 >= M || n0 >= N) return;  // quadrant outside the matrix (the whole workgroup leaves)
   }
-  // K counts elements; a row holds k_bytes bytes, a K-step is 128 of them.  With FP4 the last
-  // step may be half filled (K % 256 == 128): its second MFMA is then switched off through the
-  // scales (see scale_bits) and its loads stay inside the first 64 bytes.
+  // K counts elements (a multiple of 32, the MX block); a row holds k_bytes bytes, a K-step is 128 of
+  // them.  The last step may be partly filled.  Its loads then stay inside the row: a 16-byte chunk past
+  // the end reads a valid chunk of the same row again (tail_adj), and what it reads does not count,
+  // because its K-blocks are the zero padding of the blocked scale buffers: byte 0 on both sides scales
+  // the block's sum by 2^-254, which leaves the accumulator as it is (the re-read payload is finite
+  // unless the row holds a NaN, and then the row's results are NaN anyway).  With FP4 a step is two
+  // 128-element scale chunks; when the last step has no second chunk at all (K % 256 in 1..128) its
+  // second MFMA is switched off through the scale operand (see scale_bits).
   const int k_bytes = FP4 ? K / 2 : K;
   int k_steps = (k_bytes + kBK - 1) / kBK;
-  const int k_chunks = K / 128;                                   // blocked scale chunks per 128 rows
-  int half_step = (FP4 && (k_bytes % kBK) != 0) ? k_steps - 1 : -1;  // index of a half-filled step
+  const int k_chunks = (K + 127) / 128;                           // blocked scale chunks per 128 rows
+  int tail_step = (k_bytes % kBK) != 0 ? k_steps - 1 : -1;        // index of a partly filled step
+  int half_step = (FP4 && (k_chunks & 1)) ? k_steps - 1 : -1;     // index of a step without a second scale chunk
   // SPLIT: this workgroup walks steps ks_begin .. ks_begin + k_steps; from here on steps and scale
   // chunks count from ks_begin (the host makes sure that every split owns a step)
   int ks_begin = 0, k_chunks_left = k_chunks;
@@ -144,6 +150,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     ks_begin = split * per;
     k_steps = k_steps - ks_begin < per ? k_steps - ks_begin : per;
     half_step -= ks_begin;
+    tail_step -= ks_begin;
     k_chunks_left -= ks_begin * KC;
   }
 
@@ -155,7 +162,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   const uint8_t* const A_tile = A + (int64_t)m0 * lda + (int64_t)ks_begin * kBK;
   const uint8_t* const B_tile = B + (int64_t)n0 * ldb + (int64_t)ks_begin * kBK;
   const int lrow = lane >> 3, lchunk = (lane & 7) ^ lrow;
-  const uint32_t half_adj = (lchunk & 4) ? 64u : 0u;  // in a half-filled step chunks 4-7 re-read chunks 0-3
+  // in a partly filled step of v valid chunks, chunk c >= v reads chunk c % v again
+  const int tail_chunks = (k_bytes % kBK) / 16;
+  const uint32_t tail_adj = tail_chunks > 0 ? (uint32_t)(lchunk - lchunk % tail_chunks) * 16u : 0u;
   uint32_t offA[kLoadsA], offB[kLoadsB];
 #pragma unroll
   for (int i = 0; i < kLoadsA; ++i) {
@@ -193,7 +202,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
                  : "memory");  // M0 has no other user in this kernel (LDS reads do not need it on gfx9+)
   };
   auto fetch_one = [&](int n, int ks, uint32_t buf) {
-    const uint32_t adj = (FP4 && ks == half_step) ? half_adj : 0u;
+    const uint32_t adj = ks == tail_step ? tail_adj : 0u;
     if (n < kLoadsA) {
       dma16(A_tile + (int64_t)ks * kBK, offA[n] - adj, buf + (wave * kLoadsA + n) * kGroupStride);
     } else if (n < kLoadsA + kLoadsB) {
@@ -677,7 +686,7 @@ int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb
             dt_stream_t stream) {
   if (M < 0 || N < 0 || K < 0) return DT_ERR_INVALID_SHAPE;
   if (M == 0 || N == 0) return DT_OK;
-  if (K == 0 || K % 128 != 0) return DT_ERR_INVALID_SHAPE;  // one scaled MFMA covers 128 elements
+  if (K == 0 || K % 32 != 0) return DT_ERR_INVALID_SHAPE;  // whole MX blocks
   const int64_t k_bytes = FP4 ? K / 2 : K;
   if (N % 4 != 0 || ldo % 4 != 0 || ldo < N || lda < k_bytes || ldb < k_bytes) return DT_ERR_INVALID_SHAPE;
   if (M > 0x7FFFFF00ll || N > 0x7FFFFF00ll || K > 0x7FFFFF00ll) return DT_ERR_INVALID_SHAPE;

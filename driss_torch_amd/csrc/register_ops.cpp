@@ -340,14 +340,14 @@ Tensor mx_fp8_bf16(Tensor a, Tensor b, Tensor a_scale, Tensor b_scale) {
   const int64_t M = a.size(0), K = a.size(1), N = b.size(1);
   TORCH_CHECK(b.size(0) == K, "Incompatible matrix dimensions: a is ", M, "x", K, " but b is ", b.size(0), "x", N);
   TORCH_CHECK(N % 8 == 0, "N must be a multiple of 16 but got, ", N);
-  TORCH_CHECK(K % 128 == 0, "K must be a multiple of 128 but got ", K);
+  TORCH_CHECK(K % 32 == 0, "K must be a multiple of the MX block size 32 but got ", K);
   TORCH_CHECK(reinterpret_cast<std::uintptr_t>(a.data_ptr()) % 16 == 0, "Input tensor 'a' must be 16-byte aligned");
   TORCH_CHECK(reinterpret_cast<std::uintptr_t>(b.data_ptr()) % 16 == 0, "Input tensor 'b' must be 16-byte aligned");
-  auto ceil_div = [](int64_t x, int64_t y) { return (x + y - 1) / y; };
-  const int64_t num_k_blocks = ceil_div(K, 32);
-  const int64_t expected_a = 128 * ceil_div(M, 128) * num_k_blocks;
+  // the length of the blocked layout: 128 ceil(M / 128) rows of 4 ceil(K / 128) bytes, which is the
+  // reference's 128 ceil(M / 128) ceil(K / 32) (:197-205) whenever K is a multiple of 128
+  const int64_t expected_a = dt_blocked_scale_bytes(M, K / 32);
   TORCH_CHECK(a_scale.numel() == expected_a, "Expected a_scale_size to be ", expected_a, " but got ", a_scale.numel());
-  const int64_t expected_b = 128 * ceil_div(N, 128) * num_k_blocks;
+  const int64_t expected_b = dt_blocked_scale_bytes(N, K / 32);
   TORCH_CHECK(b_scale.numel() == expected_b, "Expected b_scale_size to be ", expected_b, " but got ", b_scale.numel());
   TORCH_CHECK(a.stride(1) == 1, "Input tensor 'a' must be contiguous in the K dimension (row-major)");
   TORCH_CHECK(b.stride(0) == 1, "Input tensor 'b' must be contiguous in the K dimension (column-major)");
@@ -384,14 +384,14 @@ Tensor mx_fp4_bf16(Tensor a, Tensor b, Tensor a_scale, Tensor b_scale) {
   const int64_t M = a.size(0), Kp = a.size(1), K = 2 * Kp, N = b.size(1);
   TORCH_CHECK(b.size(0) == Kp, "Incompatible matrix dimensions: a is ", M, "x", Kp, " but b is ", b.size(0), "x", N);
   TORCH_CHECK(N % 8 == 0, "N must be a multiple of 16 but got, ", N);
-  TORCH_CHECK(K % 128 == 0, "K must be a multiple of 128 but got ", K);
+  TORCH_CHECK(K % 32 == 0, "K must be a multiple of the MX block size 32 but got ", K);
   TORCH_CHECK(reinterpret_cast<std::uintptr_t>(a.data_ptr()) % 16 == 0, "Input tensor 'a' must be 16-byte aligned");
   TORCH_CHECK(reinterpret_cast<std::uintptr_t>(b.data_ptr()) % 16 == 0, "Input tensor 'b' must be 16-byte aligned");
-  auto ceil_div = [](int64_t x, int64_t y) { return (x + y - 1) / y; };
-  const int64_t num_k_blocks = ceil_div(K, 32);
-  const int64_t expected_a = 128 * ceil_div(M, 128) * num_k_blocks;
+  // the length of the blocked layout: 128 ceil(M / 128) rows of 4 ceil(K / 128) bytes, which is the
+  // reference's 128 ceil(M / 128) ceil(K / 32) (:197-205) whenever K is a multiple of 128
+  const int64_t expected_a = dt_blocked_scale_bytes(M, K / 32);
   TORCH_CHECK(a_scale.numel() == expected_a, "Expected a_scale_size to be ", expected_a, " but got ", a_scale.numel());
-  const int64_t expected_b = 128 * ceil_div(N, 128) * num_k_blocks;
+  const int64_t expected_b = dt_blocked_scale_bytes(N, K / 32);
   TORCH_CHECK(b_scale.numel() == expected_b, "Expected b_scale_size to be ", expected_b, " but got ", b_scale.numel());
   TORCH_CHECK(a.stride(1) == 1, "Input tensor 'a' must be contiguous in the K dimension (row-major)");
   TORCH_CHECK(b.stride(0) == 1, "Input tensor 'b' must be contiguous in the K dimension (column-major)");

@@ -215,7 +215,11 @@ DT_API int dt_to_blocked(const uint8_t* scale, int64_t R, int64_t C, uint8_t* ou
  * :168-214 (operand contract), :36-163 (GEMM).  a: e4m3fn [M,K], row stride lda bytes;
  * b: the reference's [K,N] tensor with stride(0)==1, i.e. e4m3fn [N,K] with row stride ldb
  * bytes; sfa / sfb: E8M0 in the blocked layout, dt_blocked_scale_bytes(M, K/32) and
- * (N, K/32) bytes.  K % 128 == 0, lda % 16 == 0, ldb % 16 == 0, a, b 16-byte aligned
+ * (N, K/32) bytes with the padding zero (dt_mx_fp8_quantize and dt_to_blocked write it so).  K % 32
+ * == 0 (the reference's own checks leave K % 128 == 0 only: its expected scale length
+ * 128 ceil(M/128) ceil(K/32), :197-205, equals the blocked layout's only then; here the length is
+ * dt_blocked_scale_bytes and any whole number of MX blocks is taken; the K-blocks of the padding
+ * count as zero).  lda % 16 == 0, ldb % 16 == 0, a, b 16-byte aligned
  * (:190-195), out 8-byte aligned, N % 4 == 0 and ldo % 4 == 0 (the reference asks N % 8, :187);
  * 256 rows of an operand must span less than 4 GiB (255*ld + K bytes); the operand itself
  * may be larger.                                                                         */
@@ -228,7 +232,7 @@ DT_API int dt_mx_fp8_bf16(const void* a, const void* b, const uint8_t* sfa, cons
  * src/mx_fp8_bf16.cu:243-271.  a: [M, K/2] bytes, b: [N, K/2] bytes (the reference's
  * [K/2, N] tensor with stride(0)==1), two e2m1 values per byte with the even element in
  * the low nibble; K counts elements, lda / ldb bytes.  Scales, alignment and shape
- * rules as for dt_mx_fp8_bf16 (K % 128 == 0).                                           */
+ * rules as for dt_mx_fp8_bf16 (K % 32 == 0).                                            */
 DT_API int dt_mx_fp4_bf16(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb,
                           int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, void* out,
                           int64_t ldo, dt_stream_t stream);

@@ -64,7 +64,7 @@ def test_host_validation_without_gpu():
     assert L.dt_mx_fp8_quantize_dual(fake, cabi.BF16, 128, 128, cabi.E4M3FN, 0, fake, fake, None, fake, None) == 3
     assert L.dt_mx_fp8_quantize_dual(fake + 1, cabi.BF16, 128, 128, cabi.E4M3FN, 0, fake, fake, fake, fake, None) == 4
     assert L.dt_mx_fp8_quantize_dual(None, cabi.BF16, 0, 128, cabi.E4M3FN, 0, None, None, None, None, None) == 0
-    assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 128, 128, 96, 96, 96, fake, 128, None) == 2  # K % 128
+    assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 128, 128, 80, 80, 80, fake, 128, None) == 2  # K % 32
     assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 128, 126, 128, 128, 128, fake, 126, None) == 2  # N % 4
     assert L.dt_mx_fp8_bf16(fake + 8, fake, fake, fake, 128, 128, 128, 128, 128, fake, 128, None) == 4
     assert L.dt_mx_fp8_bf16(fake, fake, None, fake, 128, 128, 128, 128, 128, fake, 128, None) == 3
@@ -76,12 +76,12 @@ def test_host_validation_without_gpu():
     assert L.dt_mx_gemm_workspace_init(None, 1 << 20, None) == 3
     assert L.dt_mx_gemm_workspace_init(fake, 512, None) == 5
     assert L.dt_mx_gemm_workspace_init(fake + 16, 1 << 20, None) == 4
-    assert L.dt_mx_fp8_bf16_ws(fake, fake, fake, fake, 128, 128, 96, 96, 96, fake, 128, fake, 1 << 20, None) == 2
+    assert L.dt_mx_fp8_bf16_ws(fake, fake, fake, fake, 128, 128, 80, 80, 80, fake, 128, fake, 1 << 20, None) == 2
     assert L.dt_mx_fp8_bf16_ws(fake, fake, fake, fake, 128, 128, 128, 128, 128, fake, 128, fake + 16, 1 << 20, None) == 4
     assert L.dt_mx_fp4_bf16_ws(fake, fake, fake, fake, 128, 128, 256, 128, 128, fake, 128, fake + 16, 1 << 20, None) == 4
     assert L.dt_mx_fp8_bf16_ws(fake, fake, fake, fake, 0, 128, 128, 128, 128, fake, 128, None, 0, None) == 0
     # e2m1 operands: K counts elements, the row strides bytes
-    assert L.dt_mx_fp4_bf16(fake, fake, fake, fake, 128, 128, 192, 96, 96, fake, 128, None) == 2  # K % 128
+    assert L.dt_mx_fp4_bf16(fake, fake, fake, fake, 128, 128, 176, 96, 96, fake, 128, None) == 2  # K % 32
     assert L.dt_mx_fp4_bf16(fake, fake, fake, fake, 128, 128, 256, 64, 128, fake, 128, None) == 2  # lda < K/2
     assert L.dt_mx_fp4_bf16(fake, fake + 8, fake, fake, 128, 128, 256, 128, 128, fake, 128, None) == 4
     assert L.dt_mx_fp4_bf16(fake, fake, fake, None, 128, 128, 256, 128, 128, fake, 128, None) == 3

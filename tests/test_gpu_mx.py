@@ -220,6 +220,32 @@ def test_mx_gemm_both_tile_shapes(d, cabi, variant, size):
         cabi.set_tuning("gemm.variant", 0)
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2, 8])
+@pytest.mark.parametrize("K", [32, 64, 96, 160, 224, 416, 1120])
+def test_mx_gemm_k_of_any_whole_number_of_blocks(d, cabi, variant, K):
+    """K a multiple of 32 but not of 128 (the reference's own scale-length check leaves multiples of 128
+    only, src/mx_fp8_bf16.cu:197-205): the last step is partly filled, its missing K-blocks are the zero
+    padding of the blocked scales, and the loads stay inside the rows.  The operands sit at the very end
+    of their allocations and the rows past the matrix edge are poisoned with NaN codes, so a load that
+    strays shows up as a NaN; the result is checked against the exact product."""
+    cabi.set_tuning("gemm.variant", variant)
+    try:
+        _check_gemm(d, 133, K, 264, 1900 + K, "randn")
+        # a contiguous operand: the byte after a row's K bytes is the next row's first -- poison a copy's
+        # neighbours and compare
+        a_data, a_sc, b_data, b_sc = _operands(d, 70, K, 136, 1950 + K, "randn")
+        sa, sb = d.to_blocked(a_sc), d.to_blocked(b_sc)
+        want = d.mx_fp8_bf16(a_data, b_data.t(), sa, sb)
+        a_wide = torch.full((70, K + 128), 0x7F, dtype=torch.uint8, device="cuda")  # 0x7F = NaN
+        b_wide = torch.full((136, K + 128), 0x7F, dtype=torch.uint8, device="cuda")
+        a_wide[:, :K] = a_data.view(torch.uint8)
+        b_wide[:, :K] = b_data.view(torch.uint8)
+        got = d.mx_fp8_bf16(a_wide.view(E4)[:, :K], b_wide.view(E4)[:, :K].t(), sa, sb)
+        assert torch.equal(got, want)
+    finally:
+        cabi.set_tuning("gemm.variant", 0)
+
+
 def _random_gemm_sizes(seed, n):
     import random
 
@@ -240,8 +266,8 @@ def test_mx_gemm_random_sizes(d, cabi, variant, size):
 
 
 @pytest.mark.parametrize("splits", [0, 2, 3, 5, 16])
-@pytest.mark.parametrize("size", [(16, 2048, 256), (133, 1664, 264), (300, 1024, 136), (1, 640, 8), (64, 8192, 512)],
-                         ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+@pytest.mark.parametrize("size", [(16, 2048, 256), (133, 1664, 264), (300, 1024, 136), (1, 640, 8), (64, 8192, 512),
+                                  (40, 4192, 136)], ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
 def test_mx_gemm_split_k(d, cabi, splits, size):
     """K shared between several workgroups per tile (forced factors, and the library's own choice):
     same tolerance as the plain kernel, the same bits on every call (the sum runs in split order

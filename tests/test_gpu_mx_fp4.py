@@ -75,8 +75,21 @@ def test_mx_fp4_gemm_both_tile_shapes(d, cabi, variant, size):
         cabi.set_tuning("gemm.variant", 0)
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("K", [32, 64, 96, 160, 224, 288, 352, 480, 1312])
+def test_mx_fp4_gemm_k_of_any_whole_number_of_blocks(d, cabi, variant, K):
+    """K a multiple of 32 but not of 128: the last 256-element step holds 1..7 blocks (its second
+    128-element half missing, partly or wholly filled); the K-blocks of the scale padding count as
+    zero and the loads stay inside the rows (the output is checked against the exact product)"""
+    cabi.set_tuning("gemm.variant", variant)
+    try:
+        _check(d, 133, K, 264, 970 + K, "randn")
+    finally:
+        cabi.set_tuning("gemm.variant", 0)
+
+
 @pytest.mark.parametrize("splits", [0, 2, 3, 4, 16])
-@pytest.mark.parametrize("size", [(16, 2048, 256), (133, 1408, 264), (40, 16512, 136)], ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+@pytest.mark.parametrize("size", [(16, 2048, 256), (133, 1408, 264), (40, 16512, 136), (24, 8288, 136)], ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
 def test_mx_fp4_gemm_split_k(d, cabi, splits, size):
     """K shared between workgroups, including a K whose last 256-element step is half filled
     (1408 = 5.5 steps, 16512 = 64.5, which the library splits by itself): the half step belongs to the last split only."""
@@ -162,7 +175,7 @@ def test_mx_fp4_gemm_argument_errors(d):
     with pytest.raises(RuntimeError):
         d.mx_fp4_bf16(A, B.t(), SA[:-1], SB)  # scale length for K = 2 * a.size(1)
     with pytest.raises(RuntimeError):
-        d.mx_fp4_bf16(A[:, :96], B[:, :96].t(), SA, SB)  # K = 192 is not a multiple of 128
+        d.mx_fp4_bf16(A[:, :88], B[:, :88].t(), SA, SB)  # K = 176 is not a whole number of MX blocks
     with pytest.raises(RuntimeError):
         d.mx_fp4_bf16(A.view(torch.float8_e4m3fn), B.t(), SA, SB)
 
