@@ -568,13 +568,24 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
   // mx_col_t_kernel) keeps them on the same rows of the transposed payload.  Measured, the first
   // is faster unless the matrix is much wider than tall (16384 x 4096 bf16: 50 vs 57 us; 4096 x
   // 16384: 53 vs 52 us; without the row-wise half the second wins from square on), so the host
-  // picks by shape.
+  // picks by shape (cols_first: 1 = the first, 0 = the second, 2 = the banded order below).
   const uint32_t row_tiles = (rows + kDualRows - 1) / kDualRows;
   uint32_t tr, tc;
-  if (cols_first) {
-    const uint32_t col_tiles = (cols + kTileCols - 1) / kTileCols;
+  const uint32_t col_tiles = (cols + kTileCols - 1) / kTileCols;
+  if (cols_first == 1) {
     tr = blockIdx.x / col_tiles;
     tc = blockIdx.x - tr * col_tiles;
+  } else if (cols_first == 2 && row_tiles % 8 == 0) {
+    // bands of 8 row tiles: inside a band 8 tiles down the rows, then on to the next column tile, so that
+    // the workgroups in flight cover whole rows of x and still write 8 adjacent pieces of an output row
+    uint32_t t = blockIdx.x;
+    if (t < (gridDim.x & ~63u)) {
+      const uint32_t xcd = t & 7u, slot = t >> 3;
+      t = (slot & ~7u) * 8u + xcd * 8u + (slot & 7u);
+    }
+    const uint32_t band = t / (8u * col_tiles), rem = t - band * 8u * col_tiles;
+    tc = rem >> 3;
+    tr = band * 8u + (rem & 7u);
   } else {
     uint32_t t = blockIdx.x;
     if (t < (gridDim.x & ~63u)) {
