@@ -290,30 +290,50 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
     uint32_t first2 = (uint32_t)first;
     asm volatile("" : "+v"(first2));
     const uint32_t stride32 = (uint32_t)stride, nvec32 = (uint32_t)nvec;
-    auto emit = [&](int k, u32x4 w) {
-      const uint32_t i = first2 + k * stride32;
-      if (i < nvec32) {
-        if constexpr (PAIR) {
-          static_assert(!PAIR || OUT == DT_E4M3FN, "the pair is e4m3fn + e5m2");
-          cast_vec_pair_finite<IN, ROUND_BF16>(w, s, out, out2, i);
-        } else {
-          cast_vec<IN, OUT, ROUND_BF16, false>(w, s, out, i);
-        }
+    auto emit_at = [&](uint32_t i, u32x4 w) {
+      if constexpr (PAIR) {
+        static_assert(!PAIR || OUT == DT_E4M3FN, "the pair is e4m3fn + e5m2");
+        cast_vec_pair_finite<IN, ROUND_BF16>(w, s, out, out2, i);
+      } else {
+        cast_vec<IN, OUT, ROUND_BF16, false>(w, s, out, i);
       }
     };
+    auto emit = [&](int k, u32x4 w) {
+      const uint32_t i = first2 + k * stride32;
+      if (i < nvec32) emit_at(i, w);
+    };
+    // A batch whose every slot lies inside for every lane of the workgroup is converted without the
+    // per-slot test: with a branch around each vector its 25-30 instructions run as one dependent chain
+    // (one wave per SIMD: nothing else fills the gaps), without it the compiler interleaves the batch
+    // (store phase of 8192 x 8192 bf16 -> one fp8 output: 13.9 us -> see bench).
+    auto whole_batch = [&](int k_last) { return block_first + (uint32_t)(kBlock - 1) + (uint32_t)k_last * stride32 < nvec32; };
 #pragma unroll
     for (int b = 0; b < kResRegVecs; b += kResBatch) {
       if ((uint32_t)b >= nk) break;
+      constexpr int kRegLast = kResRegVecs - 1;
+      if (whole_batch(b + kResBatch - 1 < kRegLast ? b + kResBatch - 1 : kRegLast)) {
 #pragma unroll
-      for (int j = 0; j < kResBatch; ++j)
-        if (b + j < kResRegVecs) emit(b + j, r[b + j]);
+        for (int j = 0; j < kResBatch; ++j)
+          if (b + j < kResRegVecs) emit_at(first2 + (uint32_t)(b + j) * stride32, r[b + j]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < kResBatch; ++j)
+          if (b + j < kResRegVecs) emit(b + j, r[b + j]);
+      }
     }
 #pragma unroll
     for (int b = 0; b < kResLdsVecs; b += kResBatch) {
       if ((uint32_t)(kResRegVecs + b) >= nk) break;
+      constexpr int kLdsLast = kResLdsVecs - 1;
+      if (whole_batch(kResRegVecs + (b + kResBatch - 1 < kLdsLast ? b + kResBatch - 1 : kLdsLast))) {
 #pragma unroll
-      for (int j = 0; j < kResBatch; ++j)
-        if (b + j < kResLdsVecs) emit(kResRegVecs + b + j, keep[(b + j) * kBlock + tid]);
+        for (int j = 0; j < kResBatch; ++j)
+          if (b + j < kResLdsVecs) emit_at(first2 + (uint32_t)(kResRegVecs + b + j) * stride32, keep[(b + j) * kBlock + tid]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < kResBatch; ++j)
+          if (b + j < kResLdsVecs) emit(kResRegVecs + b + j, keep[(b + j) * kBlock + tid]);
+      }
     }
     if constexpr (OVERFLOW) {  // the slots that were not kept: read again, the registers are free now
       for (uint32_t k0 = kResVecs; k0 < nk; k0 += kResBatch) {
