@@ -50,9 +50,9 @@ Knob g_knobs[] = {
     {"gemm.split_k", 0},
     {"gemm.tail_quads", 1},
     {"dynamic.resident", 1},
-    {"dynamic.resident_min_kib", 0},
-    {"dynamic.resident_gap_lo_kib", 12288},
-    {"dynamic.resident_gap_hi_kib", 40960},
+    {"dynamic.resident_min_kib", 32768},
+    {"dynamic.resident_gap_lo_kib", 0},
+    {"dynamic.resident_gap_hi_kib", 0},
     {"dynamic.resident_overflow", 1},
     {"dynamic.resident_spin_limit", 1 << 19},
 };

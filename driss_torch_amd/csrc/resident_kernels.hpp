@@ -546,9 +546,11 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
 template <bool PAIR>
 inline int launch_resident(const void* x, int in_dtype, int64_t numel, int out_dtype, int round_mode, void* ws, void* out,
                            void* out2, float* amax_out, float* scale_out, float fmax0, float fmax1, hipStream_t stream) {
-  // Where the two kernels win: between about 12 and 40 MiB the cast's second read of x comes out
-  // of the 256 MiB last-level cache faster than this kernel's barrier costs (32 MiB bf16: 17.0 vs
-  // 18.4 us).  Below, one launch beats two; above, the second read goes to HBM (128 MiB: 50 vs 61 us).
+  // Where the two kernels win: below about 32 MiB the cast's second read of x comes out of the 256 MiB
+  // last-level cache faster than this kernel's barrier and its launch with 144 KB of LDS cost (bf16, us,
+  // this kernel against the two, both fp8 outputs / one: 8 MiB 12.9 vs 11.3 / 12.6 vs 10.6, 16 MiB 14.9 vs
+  // 14.3 / 13.9 vs 13.1, 32 MiB 19.1 vs 19.7 / 17.4 vs 17.2, 48 MiB 22.8 vs 27.2 / 20.4 vs 23.1, 64 MiB
+  // 27.5 vs 34.0 / 24.0 vs 29.2, 96 MiB 37.7 vs 48.1 / 32.1 vs 40.6, 128 MiB 44.4 vs 61.9).
   const int64_t bytes = numel * (in_dtype == DT_F32 ? 4 : 2);
   // An earlier launch of the one-kernel path on this device gave up waiting for the whole chip (its
   // outputs are NaN): say so once, and leave the path off for the rest of the process.
