@@ -289,7 +289,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     HalfWords r;
 #pragma unroll
     for (int c = 0; c < KC; ++c) {
-      if constexpr (H == 4) {
+      if constexpr (!FP4) {
+        // e4m3: each lane reads the one byte it needs (the K-block lane / 16 of its row's word); o includes it
+        if constexpr (H == 4) {
+          r.w[c][0] = lds[o + c * 1024 + half * 8];       r.w[c][1] = lds[o + c * 1024 + 256 + half * 8];
+          r.w[c][2] = lds[o + c * 1024 + half * 8 + 4];   r.w[c][3] = lds[o + c * 1024 + 256 + half * 8 + 4];
+        } else {
+          r.w[c][0] = lds[o + c * 1024 + half * 4];
+          r.w[c][1] = lds[o + c * 1024 + 256 + half * 4];
+        }
+      } else if constexpr (H == 4) {
         const u32x2 e = *reinterpret_cast<const u32x2*>(lds + o + c * 1024 + half * 8);
         const u32x2 d = *reinterpret_cast<const u32x2*>(lds + o + c * 1024 + 256 + half * 8);
         r.w[c][0] = e.x; r.w[c][1] = d.x; r.w[c][2] = e.y; r.w[c][3] = d.y;
@@ -306,7 +315,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // as it is.
   const uint32_t scale_shift = kq * 8;
   auto scale_bits = [&](uint32_t word, int c, int step) -> int {
-    if (FP4 && c == 1) return (int)__builtin_amdgcn_ubfe(word, scale_shift, step == half_step ? 0u : 8u);
+    if constexpr (!FP4) return (int)word;
+    if (c == 1) return (int)__builtin_amdgcn_ubfe(word, scale_shift, step == half_step ? 0u : 8u);
     return (int)(word >> scale_shift);
   };
   static_assert((TM == 8 || TM == 4) && (TN == 8 || TN == 4), "wave tile is 128 or 64 rows/columns");
@@ -343,8 +353,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   const uint32_t lane_lo_a = frag_lo + (a_row0 >> 3) * kGroupStride, lane_hi_a = frag_hi + (a_row0 >> 3) * kGroupStride;
   const uint32_t lane_lo_b = frag_lo + (b_row0 >> 3) * kGroupStride, lane_hi_b = frag_hi + (b_row0 >> 3) * kGroupStride;
   // with 4 tiles per wave the wave sits in the lower or upper 8 bytes of the 16-byte scale groups
-  const uint32_t sc_lane_a = ((a_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSA + ((TM == 4 && (wm & 1)) ? 8 : 0);
-  const uint32_t sc_lane_b = ((b_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSB + ((TN == 4 && (wn & 1)) ? 8 : 0);
+  const uint32_t sc_byte = FP4 ? 0u : (uint32_t)kq;
+  const uint32_t sc_lane_a = ((a_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSA + ((TM == 4 && (wm & 1)) ? 8 : 0) + sc_byte;
+  const uint32_t sc_lane_b = ((b_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSB + ((TN == 4 && (wn & 1)) ? 8 : 0) + sc_byte;
   Frag fa[TM], fb[TN];
   int sa[KC][TM], sb[KC][TN];
   {
