@@ -159,8 +159,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // Rows past the edge re-read the last row; their products are never stored.  The tile's first
   // row goes into the 64-bit scalar base, so the 32-bit lane offsets only span the tile's rows
   // and an operand may be larger than 4 GiB.
-  const uint8_t* const A_tile = A + (int64_t)m0 * lda + (int64_t)ks_begin * kBK;
-  const uint8_t* const B_tile = B + (int64_t)n0 * ldb + (int64_t)ks_begin * kBK;
+  // The loads of a panel go out in runs of four: the instruction's immediate offset counts on both sides
+  // (global address and LDS address), so M0 and its wait state are paid once per run and the other
+  // three loads are one instruction each.  Load n of a run carries offset n * kGroupStride; its lane
+  // offset is lowered by as much, and the scalar bases by kRunBias so that no lane offset goes negative.
+  constexpr uint32_t kRun = 4, kRunBias = (kRun - 1) * kGroupStride;
+  const uint8_t* const A_tile = A + (int64_t)m0 * lda + (int64_t)ks_begin * kBK - kRunBias;
+  const uint8_t* const B_tile = B + (int64_t)n0 * ldb + (int64_t)ks_begin * kBK - kRunBias;
   const int lrow = lane >> 3, lchunk = (lane & 7) ^ lrow;
   // in a partly filled step of v valid chunks, chunk c >= v reads chunk c % v again
   const int tail_chunks = (k_bytes % kBK) / 16;
@@ -170,13 +175,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   for (int i = 0; i < kLoadsA; ++i) {
     int gr = m0 + (wave * kLoadsA + i) * kGroupRows + lrow;
     gr = gr < M ? gr : M - 1;
-    offA[i] = (uint32_t)((int64_t)(gr - m0) * lda + lchunk * 16);
+    offA[i] = (uint32_t)((int64_t)(gr - m0) * lda + lchunk * 16) + kRunBias - (i % kRun) * kGroupStride;
   }
 #pragma unroll
   for (int i = 0; i < kLoadsB; ++i) {
     int gr = n0 + (wave * kLoadsB + i) * kGroupRows + lrow;
     gr = gr < N ? gr : N - 1;
-    offB[i] = (uint32_t)((int64_t)(gr - n0) * ldb + lchunk * 16);
+    offB[i] = (uint32_t)((int64_t)(gr - n0) * ldb + lchunk * 16) + kRunBias - (i % kRun) * kGroupStride;
   }
   // Scales: KC more wave-wide loads per step.  Even waves bring A chunks, odd waves B chunks:
   // lanes 0-31 the tile's first 128-row chunk, lanes 32-63 the next one (the second chunk of a
@@ -191,33 +196,50 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   const int sc_dst = wave_is_b ? kOffSB : kOffSA;
   // load number n of a step: n < kLoadsA -> A group, < kLoadsA+kLoadsB -> B group, else scales
   constexpr int kLoadsPerStep = kLoadsA + kLoadsB + KC;
-    // global_load_lds_dwordx4 in its scalar-base + 32-bit-lane-offset form (the builtin is
+  // global_load_lds_dwordx4 in its scalar-base + 32-bit-lane-offset form (the builtin is
   // selected with a 64-bit address per lane, which costs a 64-bit add and a second address
-  // register per load); M0 carries the LDS destination.
+  // register per load); M0 carries the LDS destination of the run's first load.
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
-  auto dma16 = [&](const uint8_t* uniform_base, uint32_t lane_off, uint32_t lds_off) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(lds_base + lds_off), "v"(lane_off), "s"(uniform_base)
-                 : "memory");  // M0 has no other user in this kernel (LDS reads do not need it on gfx9+)
+  static_assert(kRun == 4 && kGroupStride == 1024, "the immediate offsets below");
+  auto dma16 = [&](int run_pos, const uint8_t* uniform_base, uint32_t lane_off, uint32_t lds_off) {
+    // M0 has no other user in this kernel (LDS reads do not need it on gfx9+)
+    if (run_pos == 0)
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                   :
+                   : "s"(lds_base + lds_off), "v"(lane_off), "s"(uniform_base)
+                   : "memory");
+    else if (run_pos == 1)
+      asm volatile("global_load_lds_dwordx4 %0, %1 offset:1024" : : "v"(lane_off), "s"(uniform_base) : "memory");
+    else if (run_pos == 2)
+      asm volatile("global_load_lds_dwordx4 %0, %1 offset:2048" : : "v"(lane_off), "s"(uniform_base) : "memory");
+    else
+      asm volatile("global_load_lds_dwordx4 %0, %1 offset:3072" : : "v"(lane_off), "s"(uniform_base) : "memory");
   };
-  auto fetch_one = [&](int n, int ks, uint32_t buf) {
-    const uint32_t adj = ks == tail_step ? tail_adj : 0u;
+  // adj: what a lane's offset gives way by in a partly filled step (the prologue passes it; in the K loop
+  // the offsets themselves are lowered once, see tail_in_place, so that a refill is one instruction)
+  auto fetch_one = [&](int n, int ks, uint32_t buf, uint32_t adj) {
     if (n < kLoadsA) {
-      dma16(A_tile + (int64_t)ks * kBK, offA[n] - adj, buf + (wave * kLoadsA + n) * kGroupStride);
+      dma16(n % kRun, A_tile + (int64_t)ks * kBK, offA[n] - adj, buf + (wave * kLoadsA + n - n % kRun) * kGroupStride);
     } else if (n < kLoadsA + kLoadsB) {
       const int i = n - kLoadsA;
-      dma16(B_tile + (int64_t)ks * kBK, offB[i] - adj, buf + kOffB + (wave * kLoadsB + i) * kGroupStride);
+      dma16(i % kRun, B_tile + (int64_t)ks * kBK, offB[i] - adj, buf + kOffB + (wave * kLoadsB + i - i % kRun) * kGroupStride);
     } else {
       const int c = n - kLoadsA - kLoadsB;  // chunk of the step; past the end it re-reads the last one (switched off)
       int kc = ks * KC + c;
       kc = kc < k_chunks_left ? kc : k_chunks_left - 1;
-      dma16(sc_base + (int64_t)kc * 512, sc_off, buf + sc_dst + c * 1024);
+      dma16(0, sc_base + (int64_t)kc * 512, sc_off, buf + sc_dst + c * 1024);
     }
+  };
+  auto tail_in_place = [&]() {
+    asm volatile("; partly filled last step: lane offsets lowered for good" ::: "memory");  // keeps this a branch
+#pragma unroll
+    for (int i = 0; i < kLoadsA; ++i) offA[i] -= tail_adj;
+#pragma unroll
+    for (int i = 0; i < kLoadsB; ++i) offB[i] -= tail_adj;
   };
   auto fetch = [&](int ks, uint32_t buf) {
 #pragma unroll
-    for (int n = 0; n < kLoadsPerStep; ++n) fetch_one(n, ks, buf);
+    for (int n = 0; n < kLoadsPerStep; ++n) fetch_one(n, ks, buf, ks == tail_step ? tail_adj : 0u);
   };
   // L2 prefetch (TOUCH).  The refill of a stage is issued one K-step before it is needed, which
   // is shorter than an L2 miss; and every panel line is an L2 miss for the first workgroup of
@@ -374,10 +396,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     }
   }
 
+  // every refill of the loop is the partly filled step (the loop clamps a refill at the last step)
+  if (tail_step >= 0 && tail_step < NST) tail_in_place();
   const uint64_t t_loop = wall_clock64();
   int slot = 0;  // ring slot of step ks
   int ks = 0;
   do {  // k_steps >= 1
+    if (ks + NST == tail_step) tail_in_place();  // from this refill on
     const uint32_t cur = slot * kStageBytes;
     slot = slot + 1 == NST ? 0 : slot + 1;
     const uint32_t nxt = slot * kStageBytes;                           // step ks+1
@@ -417,7 +442,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
       }
     };
     auto dma = [&]() {
-      if (n_dma < kLoadsPerStep) fetch_one(n_dma++, kn, cur);
+      if (n_dma < kLoadsPerStep) fetch_one(n_dma++, kn, cur, 0u);
     };
     // ---- before the bar: (lo,hi) pulls b[lo], (lo,lo) pulls a[hi], both from this step's slot
     // (a quadrant has S = HA * HB time slots; the HB fragments of a b half are requested every
@@ -706,7 +731,7 @@ int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb
   if (!aligned(out, 8) || !aligned(sfa, 4) || !aligned(sfb, 4)) return DT_ERR_MISALIGNED;
   if (workspace && !aligned(workspace, 256)) return DT_ERR_MISALIGNED;
   // per-lane byte offsets are 32 bits wide and span the rows of one tile (at most 256)
-  if (255 * lda + k_bytes > 0xFFFFFFFFll || 255 * ldb + k_bytes > 0xFFFFFFFFll) return DT_ERR_INVALID_SHAPE;
+  if (255 * lda + k_bytes + 3 * 1024 > 0xFFFFFFFFll || 255 * ldb + k_bytes + 3 * 1024 > 0xFFFFFFFFll) return DT_ERR_INVALID_SHAPE;  // + the bias of a run of loads
   const uint8_t* A = static_cast<const uint8_t*>(a);
   const uint8_t* B = static_cast<const uint8_t*>(b);
   hipStream_t s = as_hip(stream);
