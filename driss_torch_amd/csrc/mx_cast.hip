@@ -127,7 +127,10 @@ int launch_dual(const DualArgs& a) {
   if (tiles > 0x7FFFFFFFll) return kNotTaken;
   mx_dual_kernel<IN, OUT, LAYOUT><<<(unsigned)tiles, kBlock, 0, a.stream>>>(a.x, (uint32_t)a.rows, (uint32_t)a.cols, a.data_r,
                                                                            a.scale_r, a.data_c, a.scale_c,
-                                                                           tuning("mx.dual_order") >= 0 ? tuning("mx.dual_order") : (a.cols > 2 * a.rows ? 0 : 1));
+                                                                           tuning("mx.dual_order") >= 0 ? tuning("mx.dual_order")
+                                                                           : a.cols > 2 * a.rows                ? 0
+                                                                           : a.rows % (8 * kDualRows) == 0      ? 2
+                                                                                                                : 1);
   return launch_status();
 }
 template <int IN>

@@ -568,7 +568,9 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
   // mx_col_t_kernel) keeps them on the same rows of the transposed payload.  Measured, the first
   // is faster unless the matrix is much wider than tall (16384 x 4096 bf16: 50 vs 57 us; 4096 x
   // 16384: 53 vs 52 us; without the row-wise half the second wins from square on), so the host
-  // picks by shape (cols_first: 1 = the first, 0 = the second, 2 = the banded order below).
+  // picks by shape (cols_first: 1 = the first, 0 = the second, 2 = the banded order below, which is
+  // 1-2 % ahead of the first where the row count is a multiple of 8 tiles: 8192 x 8192 bf16 46.8
+  // against 47.2-47.8 us, fp32 67.1 against 67.7 us).
   const uint32_t row_tiles = (rows + kDualRows - 1) / kDualRows;
   uint32_t tr, tc;
   const uint32_t col_tiles = (cols + kTileCols - 1) / kTileCols;
