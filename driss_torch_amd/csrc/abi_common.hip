@@ -26,6 +26,8 @@ struct Knob {
 //   mx.colt_via_dual: 1 = the transposed column cast runs as the one-read kernel without its row half
 //   mx.dual_order: tile order of the one-read kernel: -1 = chosen by shape, 0 = down the rows first, 1 = along
 //                 the columns first, 2 = bands of 8 row tiles
+//   mx.colt_pipe: the transposed column cast as a grid of this many workgroups per CU that walk the tiles
+//                 with the next tile's loads in flight (0 = one workgroup per tile)
 //   mx.row_band4: 1 = row-wise MX cast with blocked scales walks 4 rows x 512 elements per wave pass
 //   gemm.variant: 0 = pick the tile by problem size, 1 = 128x128 tiles, 2 = 256x256 tiles,
 //                 7 = 256x256 tiles without the L2 prefetch loads, 8 = 256x256 tiles on 8 waves (e4m3 only)
@@ -44,6 +46,7 @@ Knob g_knobs[] = {
     {"mx.col_blocks_per_cu", 32},
     {"mx.dual", 1},
     {"mx.dual_order", -1},
+    {"mx.colt_pipe", 2},
     {"mx.colt_via_dual", 1},
     {"mx.row_band4", 1},
     {"gemm.variant", 0},

@@ -549,7 +549,9 @@ __device__ __forceinline__ uint32_t other_half_max_pk16(uint32_t v) {  // v: two
 
 // WITH_ROWS = false leaves out the row-wise half (data_r / scale_r unused): the transposed column
 // cast on its own.  cols then only has to be a multiple of a lane's kV columns.
-template <int IN, int OUT, int LAYOUT, bool WITH_ROWS = true>
+// PIPE: a grid smaller than the tile count; a workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...
+// and has the loads of its next tile in flight while it converts and stores the one in hand.
+template <int IN, int OUT, int LAYOUT, bool WITH_ROWS = true, bool PIPE = false>
 __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict__ x, uint32_t rows, uint32_t cols,
                                                          uint8_t* __restrict__ data_r, uint8_t* __restrict__ scale_r,
                                                          uint8_t* __restrict__ data_c, uint8_t* __restrict__ scale_c, int cols_first) {
@@ -572,44 +574,60 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
   // 1-2 % ahead of the first where the row count is a multiple of 8 tiles: 8192 x 8192 bf16 46.8
   // against 47.2-47.8 us, fp32 67.1 against 67.7 us).
   const uint32_t row_tiles = (rows + kDualRows - 1) / kDualRows;
-  uint32_t tr, tc;
   const uint32_t col_tiles = (cols + kTileCols - 1) / kTileCols;
-  if (cols_first == 1) {
-    tr = blockIdx.x / col_tiles;
-    tc = blockIdx.x - tr * col_tiles;
-  } else if (cols_first == 2 && row_tiles % 8 == 0) {
-    // bands of 8 row tiles: inside a band 8 tiles down the rows, then on to the next column tile, so that
-    // the workgroups in flight cover whole rows of x and still write 8 adjacent pieces of an output row
-    uint32_t t = blockIdx.x;
-    if (t < (gridDim.x & ~63u)) {
-      const uint32_t xcd = t & 7u, slot = t >> 3;
-      t = (slot & ~7u) * 8u + xcd * 8u + (slot & 7u);
-    }
-    const uint32_t band = t / (8u * col_tiles), rem = t - band * 8u * col_tiles;
-    tc = rem >> 3;
-    tr = band * 8u + (rem & 7u);
-  } else {
-    uint32_t t = blockIdx.x;
-    if (t < (gridDim.x & ~63u)) {
-      const uint32_t xcd = t & 7u, slot = t >> 3;
-      t = (slot & ~7u) * 8u + xcd * 8u + (slot & 7u);
-    }
-    tc = t / row_tiles;
-    tr = t - tc * row_tiles;
-  }
+  const uint32_t ntiles = row_tiles * col_tiles;
   const uint32_t lrow0 = w * 32 + h * 16;                      // first of this lane's 16 rows inside the tile
-  const uint32_t row0 = tr * kDualRows + lrow0, col0 = tc * kTileCols + c8 * kV;
-  const bool active = row0 < rows && col0 < cols;              // rows % 32 == 0 and cols % 32 == 0
+  auto locate = [&](uint32_t t, uint32_t& tr, uint32_t& tc) {
+    if (cols_first == 1) {
+      tr = t / col_tiles;
+      tc = t - tr * col_tiles;
+    } else if (cols_first == 2 && row_tiles % 8 == 0) {
+      // bands of 8 row tiles: inside a band 8 tiles down the rows, then on to the next column tile, so that
+      // the workgroups in flight cover whole rows of x and still write 8 adjacent pieces of an output row
+      if (t < (ntiles & ~63u)) {
+        const uint32_t xcd = t & 7u, slot = t >> 3;
+        t = (slot & ~7u) * 8u + xcd * 8u + (slot & 7u);
+      }
+      const uint32_t band = t / (8u * col_tiles), rem = t - band * 8u * col_tiles;
+      tc = rem >> 3;
+      tr = band * 8u + (rem & 7u);
+    } else {
+      if (t < (ntiles & ~63u)) {
+        const uint32_t xcd = t & 7u, slot = t >> 3;
+        t = (slot & ~7u) * 8u + xcd * 8u + (slot & 7u);
+      }
+      tc = t / row_tiles;
+      tr = t - tc * row_tiles;
+    }
+  };
+  auto load_tile = [&](uint32_t t, u32x4 (&dst)[16]) {
+    uint32_t ltr, ltc;
+    locate(t, ltr, ltc);
+    const uint32_t lr0 = ltr * kDualRows + lrow0, lc0 = ltc * kTileCols + c8 * kV;
+    if (t < ntiles && lr0 < rows && lc0 < cols) {
+      const uint8_t* p = static_cast<const uint8_t*>(x) + ((uint64_t)lr0 * cols + lc0) * kB;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) dst[i] = ld_x16<IN>(p + (uint64_t)i * cols * kB);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) dst[i] = u32x4{0u, 0u, 0u, 0u};
+    }
+  };
 
   saturate_fp8_conversions();
-  u32x4 v[16];
-  if (active) {
-    const uint8_t* p = static_cast<const uint8_t*>(x) + ((uint64_t)row0 * cols + col0) * kB;
+  u32x4 v[16], vn[PIPE ? 16 : 1];
+  if constexpr (PIPE) load_tile(blockIdx.x, vn);
+  for (uint32_t tix = blockIdx.x; tix < ntiles; tix += gridDim.x) {  // tix: number of the tile in hand
+  uint32_t tr, tc;
+  locate(tix, tr, tc);
+  const uint32_t row0 = tr * kDualRows + lrow0, col0 = tc * kTileCols + c8 * kV;
+  const bool active = row0 < rows && col0 < cols;              // rows % 32 == 0 and cols % 32 == 0
+  if constexpr (PIPE) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) v[i] = ld_x16<IN>(p + (uint64_t)i * cols * kB);
+    for (int i = 0; i < 16; ++i) v[i] = vn[i];
+    load_tile(tix + gridDim.x, vn);  // in flight under everything below
   } else {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) v[i] = u32x4{0u, 0u, 0u, 0u};
+    load_tile(tix, v);
   }
 
   // ---- blocks down the columns: maxima over this lane's 16 rows, then over both halves
@@ -734,6 +752,8 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
       }
     }
   }
+  if (tix + gridDim.x < ntiles) __syncthreads();  // the LDS tiles are written again
+  }  // tile loop
 }
 
 // ----------------------------------------- blocks along rows, transposed payload

@@ -167,6 +167,15 @@ def test_mx_cast_config4_full_size(d):
     assert ((deq.reshape(256, 256, 32) - x).abs().amax(-1) <= x.abs().amax(-1) * 2**-4).all()
 
 
+def test_mx_cast_transposed_columns_walked_tiles_ragged(d):
+    """More tiles than the transposed column cast's grid of walking workgroups, with ragged last row and
+    column tiles: every workgroup handles a second tile whose loads were in flight under its first."""
+    a = util.student_t((2080, 8200), 1011)
+    dT, sT = d.mx_fp8_quantize(a.cuda(), 32, 0, True)
+    rdT, rsT = co.mx_quantize(a, axis=0, transpose=True)
+    assert torch.equal(util.codes(sT), rsT.flatten()) and torch.equal(util.codes(dT), rdT)
+
+
 # --------------------------------------------------------------------------- MX GEMM
 def _operands(d, M, K, N, seed, dist="rand"):
     mk = util.uniform if dist == "rand" else util.normal
