@@ -504,9 +504,11 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False, phases=None):
     b_data, sfb = cabi.mx_fp8_quantize(b, 1, False, e4, cabi.SCALE_BLOCKED)
     out = torch.empty((M, N), dtype=bf16, device=dev)
     del a, b
-    # the clocks take tens of milliseconds of sustained MFMA load to settle: warm up for ~30 launches
+    # The clock under sustained MFMA load settles over some 50 ms (30 warm-up launches and 25 timed ones read
+    # 5 % slower than the steady state that 150 + 100 launches reach): the GEMM rows report the steady state.
+    GEMM_WARMUP, GEMM_STEPS = max(150, W), max(100, K // 2)
     gemm8 = bind(cabi, lambda: cabi.mx_fp8_bf16(a_data, b_data, sfa, sfb, out))
-    us = time_launches(lambda i: gemm8(), 1, max(20, K // 2), max(30, W))
+    us = time_launches(lambda i: gemm8(), 1, GEMM_STEPS, GEMM_WARMUP)
     flops = 2.0 * M * N * Kd
     tf = flops / (us * 1e-6) / 1e12
     if phases is not None:
@@ -521,7 +523,7 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False, phases=None):
     ones_a = torch.full((M, Kd), 0x38, dtype=torch.uint8, device=dev).view(e4)
     ones_s = torch.full_like(sfa, 127)
     gemm1 = bind(cabi, lambda: cabi.mx_fp8_bf16(ones_a, ones_a, ones_s, ones_s, out))
-    us1 = time_launches(lambda i: gemm1(), 1, max(20, K // 2), max(30, W))
+    us1 = time_launches(lambda i: gemm1(), 1, GEMM_STEPS, GEMM_WARMUP)
     rows.append({"kernel": "mx_fp8_bf16", "workload": "8192^3, every operand element 1.0 (same schedule and traffic, little switching power)",
                  "bound": "mfma", "avg_us": round(us1, 2), "achieved_TFLOPs": round(flops / (us1 * 1e-6) / 1e12, 1),
                  "frac_of_fp8_peak": round(flops / (us1 * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4), "flops": flops})
@@ -530,7 +532,7 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False, phases=None):
     # MFMAs, which shows on constant operands only -- on random ones the clock gives way by as much
     cabi.set_tuning("gemm.variant", 8)
     try:
-        us8 = time_launches(lambda i: gemm8(), 1, max(20, K // 2), max(30, W))
+        us8 = time_launches(lambda i: gemm8(), 1, GEMM_STEPS, GEMM_WARMUP)
     finally:
         cabi.set_tuning("gemm.variant", 0)
     rows.append({"kernel": "mx_fp8_bf16", "workload": "config 5 on 8 waves per workgroup (gemm.variant 8), same operands",
@@ -552,7 +554,7 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False, phases=None):
     a4, s4a = cabi.mx_fp4_quantize(rnd((M, Kd), bf16, 1), cabi.SCALE_BLOCKED)
     b4, s4b = cabi.mx_fp4_quantize(rnd((N, Kd), bf16, 2), cabi.SCALE_BLOCKED)
     gemm4 = bind(cabi, lambda: cabi.mx_fp4_bf16(a4, b4, s4a, s4b, out))
-    us = time_launches(lambda i: gemm4(), 1, max(20, K // 2), max(30, W))
+    us = time_launches(lambda i: gemm4(), 1, GEMM_STEPS, GEMM_WARMUP)
     tf = flops / (us * 1e-6) / 1e12
     rows.append({"kernel": "mx_fp4_bf16", "workload": "8192^3 e2m1 x e2m1, E8M0 block-32 scales -> bf16",
                  "bound": "mfma", "avg_us": round(us, 2), "achieved_TFLOPs": round(tf, 1),
