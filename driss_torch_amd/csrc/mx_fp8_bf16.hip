@@ -306,13 +306,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   struct HalfWords {
     uint32_t w[KC][4];  // [chunk of the step][tile of the half]
   };
-  auto read_half_scales = [&](auto h_tag, uint32_t o, int half) -> HalfWords {  // o: stage + operand slot + lane part
+  // BYTES (e4m3, and only for scales that are used in the basic block that loads them, i.e. in the step
+  // they belong to): each lane reads the one byte it needs, the K-block lane / 16 of its row's word, and
+  // nothing has to be shifted.  Across the loop's back edge the compiler would move the byte's zero
+  // extension to the other side, between the last MFMA of one step and the first of the next.
+  auto read_half_scales = [&](auto h_tag, uint32_t o, int half, auto bytes_tag) -> HalfWords {  // o: stage + operand slot + lane part
     constexpr int H = decltype(h_tag)::value;
+    constexpr bool BYTES = decltype(bytes_tag)::value && !FP4;
+    if constexpr (BYTES) o += kq;
     HalfWords r;
 #pragma unroll
     for (int c = 0; c < KC; ++c) {
-      if constexpr (!FP4) {
-        // e4m3: each lane reads the one byte it needs (the K-block lane / 16 of its row's word); o includes it
+      if constexpr (BYTES) {
         if constexpr (H == 4) {
           r.w[c][0] = lds[o + c * 1024 + half * 8];       r.w[c][1] = lds[o + c * 1024 + 256 + half * 8];
           r.w[c][2] = lds[o + c * 1024 + half * 8 + 4];   r.w[c][3] = lds[o + c * 1024 + 256 + half * 8 + 4];
@@ -336,11 +341,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // 2^-254, underflows to zero (e2m1 has neither infinities nor NaNs) and leaves the accumulator
   // as it is.
   const uint32_t scale_shift = kq * 8;
-  auto scale_bits = [&](uint32_t word, int c, int step) -> int {
-    if constexpr (!FP4) return (int)word;
-    if (c == 1) return (int)__builtin_amdgcn_ubfe(word, scale_shift, step == half_step ? 0u : 8u);
+  auto scale_bits = [&](uint32_t word, int c, int step) -> int {  // of a word
+    if (FP4 && c == 1) return (int)__builtin_amdgcn_ubfe(word, scale_shift, step == half_step ? 0u : 8u);
     return (int)(word >> scale_shift);
   };
+  // These scales are used on the other side of the loop's back edge, and left alone the compiler moves
+  // their shifts over there, between the last MFMA of one step and the first of the next.  An empty
+  // statement that reads the value keeps the shift (and the wait for the word) in the slot it is written in.
+  auto pin_here = [](int v) { asm volatile("" : : "v"(v)); };
   static_assert((TM == 8 || TM == 4) && (TN == 8 || TN == 4), "wave tile is 128 or 64 rows/columns");
 
   // Software pipeline.  Ring slot s holds K-step ks with ks % NST == s.  The TM x TN grid of MFMAs
@@ -360,6 +368,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // nothing else would hide those latencies.  sched_barrier pins the order (the compiler
   // otherwise sinks MFMAs below waits and barriers).
   static_assert(NST >= 2 && TM % 2 == 0 && TN % 2 == 0 && TM >= TN, "pipeline shape");
+  constexpr std::true_type kBytes{};
+  constexpr std::false_type kWords{};
   constexpr std::integral_constant<int, 0> kLo{};
   constexpr std::integral_constant<int, HA> kHiA{};
   constexpr std::integral_constant<int, HB> kHiB{};
@@ -375,13 +385,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   const uint32_t lane_lo_a = frag_lo + (a_row0 >> 3) * kGroupStride, lane_hi_a = frag_hi + (a_row0 >> 3) * kGroupStride;
   const uint32_t lane_lo_b = frag_lo + (b_row0 >> 3) * kGroupStride, lane_hi_b = frag_hi + (b_row0 >> 3) * kGroupStride;
   // with 4 tiles per wave the wave sits in the lower or upper 8 bytes of the 16-byte scale groups
-  const uint32_t sc_byte = FP4 ? 0u : (uint32_t)kq;
-  const uint32_t sc_lane_a = ((a_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSA + ((TM == 4 && (wm & 1)) ? 8 : 0) + sc_byte;
-  const uint32_t sc_lane_b = ((b_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSB + ((TN == 4 && (wn & 1)) ? 8 : 0) + sc_byte;
+  const uint32_t sc_lane_a = ((a_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSA + ((TM == 4 && (wm & 1)) ? 8 : 0);
+  const uint32_t sc_lane_b = ((b_row0 & ~127) >> 7) * 512 + l16 * 16 + kOffSB + ((TN == 4 && (wn & 1)) ? 8 : 0);
   Frag fa[TM], fb[TN];
   int sa[KC][TM], sb[KC][TN];
   {
-    const HalfWords wa = read_half_scales(kHiA, sc_lane_a, 0), wb = read_half_scales(kHiB, sc_lane_b, 1);
+    const HalfWords wa = read_half_scales(kHiA, sc_lane_a, 0, kWords), wb = read_half_scales(kHiB, sc_lane_b, 1, kWords);
 #pragma unroll
     for (int t = 0; t < HA; ++t) {
       fa[t] = load_frag(lane_lo_a, lane_hi_a, 0, t * 16);
@@ -399,17 +408,20 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // every refill of the loop is the partly filled step (the loop clamps a refill at the last step)
   if (tail_step >= 0 && tail_step < NST) tail_in_place();
   const uint64_t t_loop = wall_clock64();
-  int slot = 0;  // ring slot of step ks
+  // What a step needs of its ring slot `cur` and of the next step's `nxt`: the slots' offsets and the
+  // per-lane fragment and scale addresses in them.  They are carried from step to step (this step's
+  // `nxt` set is the next step's `cur` set) and the new `nxt` set is worked out in the middle of the
+  // step's MFMA stream: whatever sits between the last MFMA of a step and the first of the next runs
+  // with the MFMA pipe idle.
+  uint32_t cur = 0, nxt = kStageBytes;  // NST >= 2
+  uint32_t cla = lane_lo_a, cha = lane_hi_a, clb = lane_lo_b, chb = lane_hi_b, csa = sc_lane_a, csb = sc_lane_b;
   int ks = 0;
   do {  // k_steps >= 1
-    if (ks + NST == tail_step) tail_in_place();  // from this refill on
-    const uint32_t cur = slot * kStageBytes;
-    slot = slot + 1 == NST ? 0 : slot + 1;
-    const uint32_t nxt = slot * kStageBytes;                           // step ks+1
+    if (ks + NST == tail_step) tail_in_place();  // from this step's refill on
     const int kn = ks + NST < k_steps ? ks + NST : k_steps - 1;       // refill of `cur` (clamped at the end: ignored)
-    const uint32_t cla = cur + lane_lo_a, cha = cur + lane_hi_a, clb = cur + lane_lo_b, chb = cur + lane_hi_b;
-    const uint32_t nla = nxt + lane_lo_a, nha = nxt + lane_hi_a, nlb = nxt + lane_lo_b, nhb = nxt + lane_hi_b;
+    uint32_t nla, nha, nlb, nhb, nsa, nsb, nxt2;
     int n_dma = 0;
+    bool touched = false;
     HalfWords hw;  // scale words of the half a quadrant brings in
     __builtin_amdgcn_sched_barrier(0);
     // MFMAs over a tiles i0.., b tiles j0.. with the b tile as the outer index (the b half of a
@@ -449,28 +461,36 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     // HA slots, the HA fragments of an a half spread evenly over the quadrant)
     constexpr int kStepA = S / HA > 1 ? S / HA - 1 : 1;  // slots between two a fragments (4 x 4 tiles: 0, 3, 6, 9)
     quadrant(kLo, kHiB, [&](int q) {
-      if (q == 0) hw = read_half_scales(kHiB, cur + sc_lane_b, 0);
+      if (q == 1) hw = read_half_scales(kHiB, csb, 0, kBytes);  // slot 0 has a fragment request
       if (q % HA == 0) fb[q / HA] = load_frag(clb, chb, kOffB, (q / HA) * 16);
       if (q == S - 1) {
 #pragma unroll
         for (int c = 0; c < KC; ++c)
 #pragma unroll
-          for (int t = 0; t < HB; ++t) sb[c][t] = scale_bits(hw.w[c][t], c, ks);
+          for (int t = 0; t < HB; ++t) sb[c][t] = FP4 ? scale_bits(hw.w[c][t], c, ks) : (int)hw.w[c][t];
       }
     });
     quadrant(kLo, kLo, [&](int q) {
-      if (q == 0) hw = read_half_scales(kHiA, cur + sc_lane_a, 1);
+      if (q == 1) hw = read_half_scales(kHiA, csa, 1, kBytes);
       if (q % kStepA == 0 && q / kStepA < HA) fa[HA + q / kStepA] = load_frag(cla, cha, 0, (HA + q / kStepA) * 16);
       if (q == S - 1) {
 #pragma unroll
         for (int c = 0; c < KC; ++c)
 #pragma unroll
-          for (int t = 0; t < HA; ++t) sa[c][HA + t] = scale_bits(hw.w[c][t], c, ks);
+          for (int t = 0; t < HA; ++t) sa[c][HA + t] = FP4 ? scale_bits(hw.w[c][t], c, ks) : (int)hw.w[c][t];
+      }
+      if (q == S - 3) {
+        nla = nxt + lane_lo_a; nha = nxt + lane_hi_a; nlb = nxt + lane_lo_b; nhb = nxt + lane_hi_b;
+      }
+      if (q == S - 2) {
+        nsa = nxt + sc_lane_a; nsb = nxt + sc_lane_b;
+        nxt2 = nxt + kStageBytes == NST * kStageBytes ? 0u : nxt + kStageBytes;
       }
     });
     // every fragment of this step has been requested; once they are in, the slot is free
     // (the queue holds, in issue order, per step in flight its stage loads and then its touch
-    // load: all but the loads of step ks+1 and whatever precedes them may stay outstanding)
+    // load: all but the loads of step ks+1 and whatever precedes them may stay outstanding.  The
+    // touch has to stay the youngest: it misses the L2 by design, and loads complete in order)
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_waitcnt vmcnt(%0)" ::"n"((NST - 2) * kVmPerStep + kTouch) : "memory");
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
@@ -479,7 +499,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     constexpr int kFragEvery = HA > 2 ? (HB >= 4 ? 3 : 2) : 1;
     static_assert(kFirstFrag + (HA - 1) * kFragEvery < S, "the a[lo] reloads fit the quadrant");
     quadrant(kHiA, kHiB, [&](int q) {
-      if (q == 0) hw = read_half_scales(kHiA, nxt + sc_lane_a, 0);
+      if (q == 0) hw = read_half_scales(kHiA, nsa, 0, kWords);
       const int f = (q - kFirstFrag) / kFragEvery;
       if (q >= kFirstFrag && (q - kFirstFrag) % kFragEvery == 0 && f < HA) fa[f] = load_frag(nla, nha, 0, f * 16);
       else if (q >= 1) dma();
@@ -487,26 +507,39 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
 #pragma unroll
         for (int c = 0; c < KC; ++c)
 #pragma unroll
-          for (int t = 0; t < HA; ++t) sa[c][t] = scale_bits(hw.w[c][t], c, ks + 1);
+          for (int t = 0; t < HA; ++t) {
+            sa[c][t] = scale_bits(hw.w[c][t], c, ks + 1);
+            pin_here(sa[c][t]);
+          }
       }
     });
 #pragma unroll
     for (int t = 0; t < kLoadsPerStep / 2; ++t)
       if (n_dma < kLoadsPerStep / 2) dma();
+    // (the last fragment is requested well before the step ends: what is still in flight at the loop's
+    // back edge is waited for in full there)
+    constexpr int kStepB = HB >= 4 ? 3 : HA;  // slots between two b fragments
+    static_assert((HB - 1) * kStepB < S, "the b[hi] reloads fit the quadrant");
     quadrant(kHiA, kLo, [&](int q) {
-      if (q == 0) hw = read_half_scales(kHiB, nxt + sc_lane_b, 1);
-      if (q % HA == 0) fb[HB + q / HA] = load_frag(nlb, nhb, kOffB, (HB + q / HA) * 16);
+      if (q == 0) hw = read_half_scales(kHiB, nsb, 1, kWords);
+      if (q % kStepB == 0 && q / kStepB < HB) fb[HB + q / kStepB] = load_frag(nlb, nhb, kOffB, (HB + q / kStepB) * 16);
+      else if (q == S - 3 && n_dma >= kLoadsPerStep) { touch(ks + NST + kTouchAhead); touched = true; }  // inside the MFMA stream if the loads are out
       else dma();
-      if (q == S - 1) {
+      if (q == S - 2) {  // not in the last slot: what follows the step's last MFMA runs with the MFMA pipe idle
 #pragma unroll
         for (int c = 0; c < KC; ++c)
 #pragma unroll
-          for (int t = 0; t < HB; ++t) sb[c][HB + t] = scale_bits(hw.w[c][t], c, ks + 1);
+          for (int t = 0; t < HB; ++t) {
+            sb[c][HB + t] = scale_bits(hw.w[c][t], c, ks + 1);
+            pin_here(sb[c][HB + t]);
+          }
       }
     });
 #pragma unroll
     for (int t = 0; t < kLoadsPerStep; ++t) dma();
-    touch(ks + NST + kTouchAhead);
+    if (!touched) touch(ks + NST + kTouchAhead);
+    cur = nxt; nxt = nxt2;
+    cla = nla; cha = nha; clb = nlb; chb = nhb; csa = nsa; csb = nsb;
   } while (++ks < k_steps);
   // the clamped refills of the last steps may still be landing: the epilogue reuses the LDS
   // (the no-ops cover the distance an assembly-written MFMA needs before its result is read)
