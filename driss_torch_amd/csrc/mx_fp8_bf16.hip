@@ -217,17 +217,26 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   };
   // adj: what a lane's offset gives way by in a partly filled step (the prologue passes it; in the K loop
   // the offsets themselves are lowered once, see tail_in_place, so that a refill is one instruction)
-  auto fetch_one = [&](int n, int ks, uint32_t buf, uint32_t adj) {
+  // the scalar bases of a step's loads
+  struct StepBases {
+    const uint8_t *a, *b, *s[KC];
+  };
+  auto base_a = [&](int ks) { return A_tile + (int64_t)ks * kBK; };
+  auto base_b = [&](int ks) { return B_tile + (int64_t)ks * kBK; };
+  auto base_s = [&](int ks, int c) {  // chunk c of the step; past the end it re-reads the last one (switched off)
+    int kc = ks * KC + c;
+    kc = kc < k_chunks_left ? kc : k_chunks_left - 1;
+    return sc_base + (int64_t)kc * 512;
+  };
+  auto fetch_one = [&](int n, const StepBases& at, uint32_t buf, uint32_t adj) {
     if (n < kLoadsA) {
-      dma16(n % kRun, A_tile + (int64_t)ks * kBK, offA[n] - adj, buf + (wave * kLoadsA + n - n % kRun) * kGroupStride);
+      dma16(n % kRun, at.a, offA[n] - adj, buf + (wave * kLoadsA + n - n % kRun) * kGroupStride);
     } else if (n < kLoadsA + kLoadsB) {
       const int i = n - kLoadsA;
-      dma16(i % kRun, B_tile + (int64_t)ks * kBK, offB[i] - adj, buf + kOffB + (wave * kLoadsB + i - i % kRun) * kGroupStride);
+      dma16(i % kRun, at.b, offB[i] - adj, buf + kOffB + (wave * kLoadsB + i - i % kRun) * kGroupStride);
     } else {
-      const int c = n - kLoadsA - kLoadsB;  // chunk of the step; past the end it re-reads the last one (switched off)
-      int kc = ks * KC + c;
-      kc = kc < k_chunks_left ? kc : k_chunks_left - 1;
-      dma16(0, sc_base + (int64_t)kc * 512, sc_off, buf + sc_dst + c * 1024);
+      const int c = n - kLoadsA - kLoadsB;
+      dma16(0, at.s[c], sc_off, buf + sc_dst + c * 1024);
     }
   };
   auto tail_in_place = [&]() {
@@ -238,8 +247,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     for (int i = 0; i < kLoadsB; ++i) offB[i] -= tail_adj;
   };
   auto fetch = [&](int ks, uint32_t buf) {
+    StepBases at;
+    at.a = base_a(ks);
+    at.b = base_b(ks);
 #pragma unroll
-    for (int n = 0; n < kLoadsPerStep; ++n) fetch_one(n, ks, buf, ks == tail_step ? tail_adj : 0u);
+    for (int c = 0; c < KC; ++c) at.s[c] = base_s(ks, c);
+#pragma unroll
+    for (int n = 0; n < kLoadsPerStep; ++n) fetch_one(n, at, buf, ks == tail_step ? tail_adj : 0u);
   };
   // L2 prefetch (TOUCH).  The refill of a stage is issued one K-step before it is needed, which
   // is shorter than an L2 miss; and every panel line is an L2 miss for the first workgroup of
@@ -266,16 +280,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
       touch_ptr = B + (int64_t)r * ldb;
     }
   }
-  auto touch = [&](int step) {
+  auto touch_address = [&](int step) -> const uint8_t* {
+    const int kt = step < k_steps ? step : k_steps - 1;
+    return touch_ptr + (uint32_t)kt * kBK;
+  };
+  auto touch_at = [&](const uint8_t* p) {
     if constexpr (TOUCH) {
-      const int kt = step < k_steps ? step : k_steps - 1;
-      const uint8_t* p = touch_ptr + (uint32_t)kt * kBK;
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
                    :
                    : "s"(lds_base + (uint32_t)(NST * kStageBytes)), "v"(p)
                    : "memory");
     }
   };
+  auto touch = [&](int step) { touch_at(touch_address(step)); };
 
   v4f acc[TM][TN];
 #pragma unroll
@@ -374,6 +391,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   constexpr std::integral_constant<int, HA> kHiA{};
   constexpr std::integral_constant<int, HB> kHiB{};
   constexpr int S = HA * HB;  // MFMA time slots per quadrant
+  // The scale values of a half are put in place one tile per time slot, in the slots that end with
+  // kScaleLast (not the quadrant's last: what follows a step's last MFMA runs with the MFMA pipe idle),
+  // from words or bytes requested in slot kScaleRead (words: slot 0).
+  constexpr int kScaleLast = S >= 8 ? S - 2 : S - 1, kScaleRead = S >= 8 ? 1 : 0;
 #pragma unroll
   for (int p = 0; p < NST; ++p) fetch(p < k_steps ? p : k_steps - 1, (uint32_t)(p * kStageBytes));
 #pragma unroll
@@ -418,8 +439,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   int ks = 0;
   do {  // k_steps >= 1
     if (ks + NST == tail_step) tail_in_place();  // from this step's refill on
-    const int kn = ks + NST < k_steps ? ks + NST : k_steps - 1;       // refill of `cur` (clamped at the end: ignored)
     uint32_t nla, nha, nlb, nhb, nsa, nsb, nxt2;
+    // the bases of step ks + NST, the refill of `cur` (clamped at the end: ignored), and the address of
+    // the touch: scalar bookkeeping of the step's second half, done in slots of the first quadrant
+    // that have nothing else to do, one item per slot
+    StepBases at;
+    const uint8_t* touch_p;
+    constexpr int kBook = S >= 8 ? 2 : S - 2;  // first of those slots (a short quadrant takes it all in one)
+    constexpr int kBookStep = S >= 8 ? 1 : 0;
     int n_dma = 0;
     bool touched = false;
     HalfWords hw;  // scale words of the half a quadrant brings in
@@ -454,30 +481,33 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
       }
     };
     auto dma = [&]() {
-      if (n_dma < kLoadsPerStep) fetch_one(n_dma++, kn, cur, 0u);
+      if (n_dma < kLoadsPerStep) fetch_one(n_dma++, at, cur, 0u);
     };
     // ---- before the bar: (lo,hi) pulls b[lo], (lo,lo) pulls a[hi], both from this step's slot
     // (a quadrant has S = HA * HB time slots; the HB fragments of a b half are requested every
     // HA slots, the HA fragments of an a half spread evenly over the quadrant)
     constexpr int kStepA = S / HA > 1 ? S / HA - 1 : 1;  // slots between two a fragments (4 x 4 tiles: 0, 3, 6, 9)
     quadrant(kLo, kHiB, [&](int q) {
-      if (q == 1) hw = read_half_scales(kHiB, csb, 0, kBytes);  // slot 0 has a fragment request
+      if (q == kScaleRead) hw = read_half_scales(kHiB, csb, 0, kBytes);  // slot 0 has a fragment request
+      const int kn = ks + NST < k_steps ? ks + NST : k_steps - 1;
+      if (q == kBook) { at.a = base_a(kn); asm volatile("" : : "s"(at.a)); }
+      if (q == kBook + kBookStep) { at.b = base_b(kn); asm volatile("" : : "s"(at.b)); }
+#pragma unroll
+      for (int c = 0; c < KC; ++c)
+        if (q == kBook + (2 + c) * kBookStep) { at.s[c] = base_s(kn, c); asm volatile("" : : "s"(at.s[c])); }
+      if (TOUCH && q == kBook + (2 + KC) * kBookStep) { touch_p = touch_address(ks + NST + kTouchAhead); asm volatile("" : : "v"(touch_p)); }
       if (q % HA == 0) fb[q / HA] = load_frag(clb, chb, kOffB, (q / HA) * 16);
-      if (q == S - 1) {
+      if (const int t = q - (kScaleLast - HB + 1); t >= 0 && t < HB) {
 #pragma unroll
-        for (int c = 0; c < KC; ++c)
-#pragma unroll
-          for (int t = 0; t < HB; ++t) sb[c][t] = FP4 ? scale_bits(hw.w[c][t], c, ks) : (int)hw.w[c][t];
+        for (int c = 0; c < KC; ++c) sb[c][t] = FP4 ? scale_bits(hw.w[c][t], c, ks) : (int)hw.w[c][t];
       }
     });
     quadrant(kLo, kLo, [&](int q) {
-      if (q == 1) hw = read_half_scales(kHiA, csa, 1, kBytes);
+      if (q == kScaleRead) hw = read_half_scales(kHiA, csa, 1, kBytes);
       if (q % kStepA == 0 && q / kStepA < HA) fa[HA + q / kStepA] = load_frag(cla, cha, 0, (HA + q / kStepA) * 16);
-      if (q == S - 1) {
+      if (const int t = q - (kScaleLast - HA + 1); t >= 0 && t < HA) {
 #pragma unroll
-        for (int c = 0; c < KC; ++c)
-#pragma unroll
-          for (int t = 0; t < HA; ++t) sa[c][HA + t] = FP4 ? scale_bits(hw.w[c][t], c, ks) : (int)hw.w[c][t];
+        for (int c = 0; c < KC; ++c) sa[c][HA + t] = FP4 ? scale_bits(hw.w[c][t], c, ks) : (int)hw.w[c][t];
       }
       if (q == S - 3) {
         nla = nxt + lane_lo_a; nha = nxt + lane_hi_a; nlb = nxt + lane_lo_b; nhb = nxt + lane_hi_b;
@@ -503,14 +533,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
       const int f = (q - kFirstFrag) / kFragEvery;
       if (q >= kFirstFrag && (q - kFirstFrag) % kFragEvery == 0 && f < HA) fa[f] = load_frag(nla, nha, 0, f * 16);
       else if (q >= 1) dma();
-      if (q == S - 1) {
+      if (const int t = q - (kScaleLast - HA + 1); t >= 0 && t < HA) {
 #pragma unroll
-        for (int c = 0; c < KC; ++c)
-#pragma unroll
-          for (int t = 0; t < HA; ++t) {
-            sa[c][t] = scale_bits(hw.w[c][t], c, ks + 1);
-            pin_here(sa[c][t]);
-          }
+        for (int c = 0; c < KC; ++c) {
+          sa[c][t] = scale_bits(hw.w[c][t], c, ks + 1);
+          pin_here(sa[c][t]);
+        }
       }
     });
 #pragma unroll
@@ -523,21 +551,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     quadrant(kHiA, kLo, [&](int q) {
       if (q == 0) hw = read_half_scales(kHiB, nsb, 1, kWords);
       if (q % kStepB == 0 && q / kStepB < HB) fb[HB + q / kStepB] = load_frag(nlb, nhb, kOffB, (HB + q / kStepB) * 16);
-      else if (q == S - 3 && n_dma >= kLoadsPerStep) { touch(ks + NST + kTouchAhead); touched = true; }  // inside the MFMA stream if the loads are out
+      else if (q == S - 3 && n_dma >= kLoadsPerStep) { touch_at(touch_p); touched = true; }  // inside the MFMA stream if the loads are out
       else dma();
-      if (q == S - 2) {  // not in the last slot: what follows the step's last MFMA runs with the MFMA pipe idle
+      if (const int t = q - (kScaleLast - HB + 1); t >= 0 && t < HB) {
 #pragma unroll
-        for (int c = 0; c < KC; ++c)
-#pragma unroll
-          for (int t = 0; t < HB; ++t) {
-            sb[c][HB + t] = scale_bits(hw.w[c][t], c, ks + 1);
-            pin_here(sb[c][HB + t]);
-          }
+        for (int c = 0; c < KC; ++c) {
+          sb[c][HB + t] = scale_bits(hw.w[c][t], c, ks + 1);
+          pin_here(sb[c][HB + t]);
+        }
       }
     });
 #pragma unroll
     for (int t = 0; t < kLoadsPerStep; ++t) dma();
-    if (!touched) touch(ks + NST + kTouchAhead);
+    if (!touched) touch_at(touch_p);
     cur = nxt; nxt = nxt2;
     cla = nla; cha = nha; clb = nlb; chb = nhb; csa = nsa; csb = nsb;
   } while (++ks < k_steps);
