@@ -528,16 +528,6 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False, phases=None):
                  "bound": "mfma", "avg_us": round(us1, 2), "achieved_TFLOPs": round(flops / (us1 * 1e-6) / 1e12, 1),
                  "frac_of_fp8_peak": round(flops / (us1 * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4), "flops": flops})
     del ones_a, ones_s
-    # the same tile on 8 waves, two per SIMD (gemm.variant 8): one wave's fragment reads hide behind the other's
-    # MFMAs, which shows on constant operands only -- on random ones the clock gives way by as much
-    cabi.set_tuning("gemm.variant", 8)
-    try:
-        us8 = time_launches(lambda i: gemm8(), 1, GEMM_STEPS, GEMM_WARMUP)
-    finally:
-        cabi.set_tuning("gemm.variant", 0)
-    rows.append({"kernel": "mx_fp8_bf16", "workload": "config 5 on 8 waves per workgroup (gemm.variant 8), same operands",
-                 "bound": "mfma", "avg_us": round(us8, 2), "achieved_TFLOPs": round(flops / (us8 * 1e-6) / 1e12, 1),
-                 "frac_of_fp8_peak": round(flops / (us8 * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4), "flops": flops})
     # two shapes off the 8192^3 grid, on row slices of the same operands (blocked scales are
     # stored by 128-row chunks, so a row prefix of the operand owns a prefix of its scales)
     for m_rows, n_rows, what in ((16, 8192, "16 rows: K shared between 4 workgroups per 128x128 tile"),

@@ -30,7 +30,7 @@ struct Knob {
 //                 with the next tile's loads in flight (0 = one workgroup per tile)
 //   mx.row_band4: 1 = row-wise MX cast with blocked scales walks 4 rows x 512 elements per wave pass
 //   gemm.variant: 0 = pick the tile by problem size, 1 = 128x128 tiles, 2 = 256x256 tiles,
-//                 7 = 256x256 tiles without the L2 prefetch loads, 8 = 256x256 tiles on 8 waves (e4m3 only)
+//                 7 = 256x256 tiles without the L2 prefetch loads
 //   gemm.tail_quads: 1 = tiles left over after whole rounds of 256x256 tiles run as 128x128 quadrants
 //                 or 256x128 halves when those fit the chip at once, 0 = never, 2 = always as
 //                 quadrants, 3 = always as halves

@@ -798,11 +798,6 @@ int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb
   const int64_t tiles256 = ceil_div(M, 256) * ceil_div(N, 256);
   const bool big = variant == 2 || variant == 7 || (variant == 0 && tiles256 >= device_facts().cu_count / 2);
   // <tile M, tile N, waves M, waves N, LDS ring slots, e2m1 operands>
-  // 8 waves of 128 x 64 (two per SIMD, so that one wave's LDS reads overlap the other's MFMAs): 74% of
-  // peak on constant data against 72%, no faster on random data, where the clock gives way first
-  if constexpr (!FP4) {
-    if (variant == 8) return launch_gemm<256, 256, 2, 4, 2, false, true>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
-  }
   if (big && variant == 7) return launch_gemm<256, 256, 2, 2, 2, FP4, false>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
   // Between a quarter and half a round of 256 x 256 tiles: as 256 x 128 halves they fill the chip
   // once (0.8 of a round of tiles), as 128 x 128 tiles they would take two rounds (2 x 0.55)
