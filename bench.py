@@ -171,8 +171,8 @@ def main():
     # ------------------------------------------------------------ headline step: config 2
     R = C = 8192
     numel = R * C
-    # Bytes of the step.  The survey's per-unit figure for the path counts x twice (one read for the
-    # reduction, one for the cast: 6 B per element with two fp8 outputs); the step's one kernel keeps
+    # Bytes of the step.  A two-kernel formulation of the path reads x twice (once for the
+    # reduction, once for the cast: 6 B per element with two fp8 outputs); the step's one kernel keeps
     # x on the chip between its passes, so what it must move -- and what the counters see -- is one
     # read of x and the two fp8 outputs: 4 B per element.  `value` and the roofline are quoted on
     # those 4 B; the 6 B figure is reported beside them as the two-pass equivalent.
@@ -263,7 +263,7 @@ def main():
         # achieved = the bytes the kernel must move (x once + two fp8 outputs: 4 B per element, its lower
         # bound) / average launch time, so frac is a fraction of the HBM peak and cannot exceed 1.  `traffic`
         # is what rocprofv3 FETCH_SIZE + WRITE_SIZE saw per launch (scaled by a plain copy), read from the
-        # committed summary of those runs.  The survey's 6 B per element (x read by the reduction and again
+        # committed summary of those runs.  The two-pass figure of 6 B per element (x read by the reduction and again
         # by the cast, as two kernels would) over the same time is two_pass_equivalent_GBs.
         "roofline": {"kernel": "resident_quant_kernel<bf16, e4m3fn+e5m2 pair>", "bound": "hbm", "achieved": round(step_gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(step_gbs / HBM_PEAK_GBS, 4),
