@@ -144,6 +144,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--gemm-only", action="store_true",
                     help="run only the block-scaled GEMM rows of the per-kernel table (for profiling) and print them")
+    ap.add_argument("--gemm-ramp", action="store_true",
+                    help="print how the 8192^3 block-scaled GEMM's launch time settles after a pause (windows of 25 launches)")
     ap.add_argument("--phases", action="store_true",
                     help="also report the per-phase times of the step's kernel (shader clock counter readings it dumps)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -162,6 +164,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     K, W = args.steps, args.warmup
+    if args.gemm_ramp:
+        print(json.dumps(gemm_ramp(torch, cabi, dev)))
+        return
     if args.gemm_only:
         ph = {} if args.phases else None
         rows = extra_kernels(torch, cabi, dev, K, W, gemm_only=True, phases=ph)
@@ -342,6 +347,45 @@ def kernel_phases(torch, cabi, launch, names, launches=20):
     out["launches"] = len(rows)
     out["unit"] = "us (100 MHz counter, 0.01 us resolution)"
     return out
+
+
+def gemm_ramp(torch, cabi, dev, windows=24, per_window=25):
+    """Launch time of the config-5 GEMM in consecutive windows of `per_window` launches, first after a
+    stretch of HBM-bound kernels (what precedes the GEMM rows in the default run), then after two seconds
+    of idling: the shader clock under sustained MFMA load needs on the order of a hundred launches to
+    settle, which is why the GEMM rows of the per-kernel table warm up with 150 launches."""
+    import time
+
+    e4, bf16 = torch.float8_e4m3fn, torch.bfloat16
+    M = N = Kd = 8192
+    g = torch.Generator().manual_seed(7)
+    a = torch.randn((M, Kd), generator=g).to(bf16).to(dev)
+    b = torch.randn((N, Kd), generator=g).to(bf16).to(dev)
+    a_data, sfa = cabi.mx_fp8_quantize(a, 1, False, e4, cabi.SCALE_BLOCKED)
+    b_data, sfb = cabi.mx_fp8_quantize(b, 1, False, e4, cabi.SCALE_BLOCKED)
+    out = torch.empty((M, N), dtype=bf16, device=dev)
+    gemm = bind(cabi, lambda: cabi.mx_fp8_bf16(a_data, b_data, sfa, sfb, out))
+    amax = bind(cabi, lambda: cabi.amax(a))
+
+    def train():
+        ev = _events(windows + 1)
+        ev[0].record()
+        for w in range(windows):
+            for _ in range(per_window):
+                gemm()
+            ev[w + 1].record()
+        torch.cuda.synchronize()
+        return [round(ev[w].elapsed_time(ev[w + 1]) * 1e3 / per_window, 1) for w in range(windows)]
+
+    gemm()
+    for _ in range(300):
+        amax()
+    torch.cuda.synchronize()
+    after_hbm = train()
+    time.sleep(2.0)
+    after_idle = train()
+    return {"kernel": "mx_fp8_bf16", "workload": "config 5: 8192^3 e4m3, N(0,1)-derived operands", "launches_per_window": per_window,
+            "us_per_launch_after_300_amax_launches": after_hbm, "us_per_launch_after_2s_idle": after_idle}
 
 
 def gemm_timeline(torch, cabi, launch, launches=5):
