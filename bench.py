@@ -222,7 +222,9 @@ def main():
 
     # timed region 2: the step is one kernel (the tensor fits the chip, see resident_kernels.hpp):
     # K launches between one pair of HIP events on the launch stream -> `roofline`
-    step_us = time_launches(step, ns, K, W)
+    # (the median of five such trains: a train of K launches lasts about 2 ms, and one hiccup of the launching
+    # thread in it shifts its average by several percent)
+    step_us = statistics.median(time_launches(step, ns, K, W) for _ in range(5))
     step_gbs = step_bytes / (step_us * 1e-6) / 1e9
 
     phases = None
