@@ -483,6 +483,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     auto dma = [&]() {
       if (n_dma < kLoadsPerStep) fetch_one(n_dma++, at, cur, 0u);
     };
+    // e4m3: the step's loads (stage refill, then the touch as the youngest) are spread evenly over the 2 S
+    // slots behind the bar: a wave gets one such load out per 40-odd cycles, so two of them in neighbouring
+    // slots of 32 cycles hold the second one's slot up (issued in runs of two to five they cost 120 cycles a
+    // step).  e2m1 keeps them out of the slots that request a fragment instead (measured both ways).
+    auto vm_ops_of_slot = [&](int slot) {  // slot: 0 .. 2 S - 1
+#pragma unroll
+      for (int i = 0; i < kVmPerStep; ++i) {
+        if ((i * 2 * S) / kVmPerStep != slot) continue;
+        if (i < kLoadsPerStep) dma();
+        else { touch_at(touch_p); touched = true; }
+      }
+    };
     // ---- before the bar: (lo,hi) pulls b[lo], (lo,lo) pulls a[hi], both from this step's slot
     // (a quadrant has S = HA * HB time slots; the HB fragments of a b half are requested every
     // HA slots, the HA fragments of an a half spread evenly over the quadrant)
@@ -531,8 +543,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     quadrant(kHiA, kHiB, [&](int q) {
       if (q == 0) hw = read_half_scales(kHiA, nsa, 0, kWords);
       const int f = (q - kFirstFrag) / kFragEvery;
-      if (q >= kFirstFrag && (q - kFirstFrag) % kFragEvery == 0 && f < HA) fa[f] = load_frag(nla, nha, 0, f * 16);
-      else if (q >= 1) dma();
+      const bool frag_slot = q >= kFirstFrag && (q - kFirstFrag) % kFragEvery == 0 && f < HA;
+      if (frag_slot) fa[f] = load_frag(nla, nha, 0, f * 16);
+      if constexpr (!FP4) vm_ops_of_slot(q);
+      else if (!frag_slot && q >= 1) dma();  // e2m1: two free issue slots per MFMA, so never next to a fragment request
       if (const int t = q - (kScaleLast - HA + 1); t >= 0 && t < HA) {
 #pragma unroll
         for (int c = 0; c < KC; ++c) {
@@ -541,17 +555,17 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
         }
       }
     });
-#pragma unroll
-    for (int t = 0; t < kLoadsPerStep / 2; ++t)
-      if (n_dma < kLoadsPerStep / 2) dma();
     // (the last fragment is requested well before the step ends: what is still in flight at the loop's
     // back edge is waited for in full there)
     constexpr int kStepB = HB >= 4 ? 3 : HA;  // slots between two b fragments
     static_assert((HB - 1) * kStepB < S, "the b[hi] reloads fit the quadrant");
     quadrant(kHiA, kLo, [&](int q) {
       if (q == 0) hw = read_half_scales(kHiB, nsb, 1, kWords);
-      if (q % kStepB == 0 && q / kStepB < HB) fb[HB + q / kStepB] = load_frag(nlb, nhb, kOffB, (HB + q / kStepB) * 16);
-      else if (q == S - 3 && n_dma >= kLoadsPerStep) { touch_at(touch_p); touched = true; }  // inside the MFMA stream if the loads are out
+      const bool frag_slot = q % kStepB == 0 && q / kStepB < HB;
+      if (frag_slot) fb[HB + q / kStepB] = load_frag(nlb, nhb, kOffB, (HB + q / kStepB) * 16);
+      if constexpr (!FP4) vm_ops_of_slot(S + q);
+      else if (frag_slot) {}
+      else if (q == S - 3 && n_dma >= kLoadsPerStep) { touch_at(touch_p); touched = true; }
       else dma();
       if (const int t = q - (kScaleLast - HB + 1); t >= 0 && t < HB) {
 #pragma unroll
