@@ -608,6 +608,15 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False, phases=None):
     rows.append({"kernel": "mx_fp4_bf16", "workload": "8192^3 e2m1 x e2m1, E8M0 block-32 scales -> bf16",
                  "bound": "mfma", "avg_us": round(us, 2), "achieved_TFLOPs": round(tf, 1),
                  "frac_of_fp4_peak": round(tf / FP4_PEAK_TFLOPS, 4), "flops": flops})
+    # 16 rows of the same operands: one pass over B (its payload and scale bytes are the algorithmic
+    # bytes; one operand set, 33 MB, so the memory-side cache may hold it); the library's kernel for few rows
+    ops4 = (a4[:16], b4, s4a[:128 * (Kd // 32)], s4b, out[:16])
+    gemm4s = bind(cabi, lambda: cabi.mx_fp4_bf16(*ops4))
+    us = time_launches(lambda i: gemm4s(), 1, max(20, K // 2), 10)
+    nbytes = N * Kd // 2 + N * Kd // 32
+    rows.append({"kernel": "mx_fp4_bf16", "workload": f"16x{N}x{Kd} e2m1 (few rows: 32 columns per workgroup, K shared between its "
+                 "eight waves, operands straight from memory into registers)", "bound": "hbm", "avg_us": round(us, 2),
+                 "achieved_GBs": round(nbytes / us / 1e3, 1), "algorithmic_bytes": nbytes, "buffer_sets": 1})
     return rows
 
 

@@ -30,13 +30,16 @@ struct Knob {
 //                 with the next tile's loads in flight (0 = one workgroup per tile)
 //   mx.row_band4: 1 = row-wise MX cast with blocked scales walks 4 rows x 512 elements per wave pass
 //   gemm.variant: 0 = pick the tile by problem size, 1 = 128x128 tiles, 2 = 256x256 tiles,
-//                 7 = 256x256 tiles without the L2 prefetch loads
+//                 7 = 256x256 tiles without the L2 prefetch loads, 9 = the kernel for at most 64 rows
+//                 whatever the other dimensions
+//   gemm.few_rows_tiles: 16-column tiles per wave of that kernel: 0 = by the number of columns, 1, 2
 //   gemm.tail_quads: 1 = tiles left over after whole rounds of 256x256 tiles run as 128x128 quadrants
 //                 or 256x128 halves when those fit the chip at once, 0 = never, 2 = always as
 //                 quadrants, 3 = always as halves
 //   gemm.split_k: 0 = share K between workgroups when the 128x128 tiling leaves CUs idle (needs the
 //                 workspace of the _ws entry points), 1 = never, n = n workgroups per tile
 Knob g_knobs[] = {
+    {"gemm.few_rows_tiles", 0},
     {"amax.blocks_per_cu", 1},
     {"amax.stream_before_cast", 0},
     {"cast.blocks_per_cu", 1},

@@ -255,6 +255,42 @@ def test_mx_gemm_k_of_any_whole_number_of_blocks(d, cabi, variant, K):
         cabi.set_tuning("gemm.variant", 0)
 
 
+@pytest.mark.parametrize("size", [(1, 640, 8), (16, 2048, 256), (17, 96, 2056), (33, 1120, 264), (48, 416, 136), (64, 8192, 512),
+                                  (5, 32, 24), (64, 160, 16)], ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+def test_mx_gemm_few_rows_kernel(d, cabi, size):
+    """the kernel for problems of at most 64 rows (16 columns per workgroup, K shared between its eight
+    waves, operands straight from memory): every count of 16-row tiles, ragged M and N, K with a partly
+    filled last 128-element step; forced here for every N, and checked against the exact product"""
+    cabi.set_tuning("gemm.variant", 9)
+    try:
+        _check_gemm(d, *size, 2100 + size[0], "randn")
+    finally:
+        cabi.set_tuning("gemm.variant", 0)
+
+
+def test_mx_gemm_few_rows_kernel_is_the_default_and_respects_strides(d, cabi):
+    """with enough columns the library takes that kernel by itself; operands and output that are slices of
+    wider tensors give the same bits, loads stay inside the rows (poisoned neighbours) and nothing is
+    written outside the output"""
+    M, K, N = 5, 4128, 4104
+    out, _ = _check_gemm(d, M, K, N, 2200, "randn")
+    cabi.set_tuning("gemm.variant", 9)
+    try:
+        a_data, a_sc, b_data, b_sc = _operands(d, M, K, N, 2200, "randn")
+        sa, sb = d.to_blocked(a_sc), d.to_blocked(b_sc)
+        assert torch.equal(d.mx_fp8_bf16(a_data, b_data.t(), sa, sb), out)
+        a_wide = torch.full((M, K + 384), 0x7F, dtype=torch.uint8, device="cuda")  # 0x7F = NaN
+        b_wide = torch.full((N, K + 640), 0x7F, dtype=torch.uint8, device="cuda")
+        a_wide[:, 128:128 + K] = a_data.view(torch.uint8)
+        b_wide[:, 256:256 + K] = b_data.view(torch.uint8)
+        out_wide = torch.full((M, N + 24), 7.0, dtype=torch.bfloat16, device="cuda")
+        cabi.mx_fp8_bf16(a_wide.view(E4)[:, 128:128 + K], b_wide.view(E4)[:, 256:256 + K], sa, sb, out_wide[:, 8:8 + N])
+        assert torch.equal(out_wide[:, 8:8 + N], out)
+        assert (out_wide[:, :8] == 7.0).all() and (out_wide[:, 8 + N:] == 7.0).all()
+    finally:
+        cabi.set_tuning("gemm.variant", 0)
+
+
 def _random_gemm_sizes(seed, n):
     import random
 

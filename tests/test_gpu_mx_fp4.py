@@ -88,6 +88,20 @@ def test_mx_fp4_gemm_k_of_any_whole_number_of_blocks(d, cabi, variant, K):
         cabi.set_tuning("gemm.variant", 0)
 
 
+@pytest.mark.parametrize("size", [(1, 640, 8), (16, 2048, 256), (17, 96, 2056), (33, 1312, 264), (48, 480, 136), (64, 8192, 512),
+                                  (5, 32, 24), (24, 4128, 4104)], ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+def test_mx_fp4_gemm_few_rows_kernel(d, cabi, size):
+    """the kernel for problems of at most 64 rows, forced for every N (the last size takes it by default
+    too): every count of 16-row tiles, ragged M and N, K with a partly filled last 128-element step"""
+    cabi.set_tuning("gemm.variant", 9)
+    try:
+        out = _check(d, *size, 2300 + size[0], "randn")
+    finally:
+        cabi.set_tuning("gemm.variant", 0)
+    if size[2] >= 4096:
+        assert torch.equal(_check(d, *size, 2300 + size[0], "randn"), out)
+
+
 @pytest.mark.parametrize("splits", [0, 2, 3, 4, 16])
 @pytest.mark.parametrize("size", [(16, 2048, 256), (133, 1408, 264), (40, 16512, 136), (24, 8288, 136)], ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
 def test_mx_fp4_gemm_split_k(d, cabi, splits, size):
