@@ -769,7 +769,9 @@ __global__ __launch_bounds__(512) void mx_skinny_kernel(const uint8_t* __restric
                                                         int M, int N, int K, int64_t lda, int64_t ldb,
                                                         uint16_t* __restrict__ out, int64_t ldo) {
   constexpr int kWavesK = 8;
-  constexpr int U = (MT == 1 || (NT == 2 && MT == 2)) ? 2 : 1;  // K-steps per batch of loads
+  // K-steps per batch of loads: what the registers hold twice over with two workgroups on a CU where the
+  // grid has that many
+  constexpr int U = MT == 1 ? (FP4 ? 4 : 2) : (NT == 2 && MT == 2) ? 2 : 1;
   constexpr int kStepBytes = FP4 ? 64 : 128;   // bytes of a row that one MFMA takes
   static_assert(MT >= 1 && MT <= 4 && NT >= 1 && MT * NT <= kWavesK, "at most 64 rows of A; one wave per output tile at the end");
   __shared__ v4f part[kWavesK][MT * NT][kWave];
