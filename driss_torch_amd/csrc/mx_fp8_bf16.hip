@@ -659,15 +659,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // 256-byte row segments.  The loop's last barrier has already retired every panel read.
   constexpr int kEpiPitch = WN * 2 + 16;
   uint8_t* epi = lds + wave * (WM * kEpiPitch);
+  // rows 16 i0 .. 16 i1 of the wave's tile: convert and park
+  auto park_rows = [&](int i0, int i1) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+    for (int i = i0; i < i1; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      u32x2 w;
-      w.x = pack_bf16x2(acc[i][j].x, acc[i][j].y);
-      w.y = pack_bf16x2(acc[i][j].z, acc[i][j].w);
-      *reinterpret_cast<u32x2*>(epi + (i * 16 + l16) * kEpiPitch + (j * 16 + kq * 4) * 2) = w;
-    }
+      for (int j = 0; j < TN; ++j) {
+        u32x2 w;
+        w.x = pack_bf16x2(acc[i][j].x, acc[i][j].y);
+        w.y = pack_bf16x2(acc[i][j].z, acc[i][j].w);
+        *reinterpret_cast<u32x2*>(epi + (i * 16 + l16) * kEpiPitch + (j * 16 + kq * 4) * 2) = w;
+      }
+  };
   constexpr int kChunksPerRow = WN * 2 / 16;             // 16-byte chunks per tile row
   constexpr int kRowsPerPass = kWave / kChunksPerRow;    // rows one store instruction covers
   const int erow = lane / kChunksPerRow, echunk = lane % kChunksPerRow;
@@ -675,13 +678,27 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // a tile wholly inside the matrix with an aligned output (the common case): no edge tests, the
   // row pointer moves by a constant
   if (wide_stores && m0 + BM <= M && n0 + BN <= N) {
+    // one 16-row strip of the wave's tile at a time, so that a strip's stores are on their way while the
+    // next one is converted (a wave only touches its own region: no barrier, the LDS counter orders the
+    // reads behind the writes).  8192^3, us per launch on constant / random operands: all rows parked
+    // first 278.3 / 380.6, in halves 276.0 / -, in quarters 274.8 / 377.8, by strips 274.3 / 376.2
+    // (without any epilogue the launch takes 259 / 352: 12 of those 19 us are the stores)
     uint16_t* dst = out + (int64_t)(m0 + wm * WM + erow) * ldo + n;
     const int64_t pass_stride = (int64_t)kRowsPerPass * ldo;
     const uint8_t* src = epi + erow * kEpiPitch + echunk * 16;
+    constexpr int kEpiParts = TM;
+    constexpr int kHalfTiles = TM / kEpiParts, kHalfRows = WM / kEpiParts;
+    static_assert(kHalfRows % kRowsPerPass == 0, "a store pass stays inside a part");
 #pragma unroll
-    for (int r = 0; r < WM; r += kRowsPerPass) {
-      *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(src + r * kEpiPitch);
-      dst += pass_stride;
+    for (int half = 0; half < kEpiParts; ++half) {
+      park_rows(half * kHalfTiles, (half + 1) * kHalfTiles);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = half * kHalfRows; r < (half + 1) * kHalfRows; r += kRowsPerPass) {
+        *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(src + r * kEpiPitch);
+        dst += pass_stride;
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (phase_log) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -694,6 +711,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     }
     return;
   }
+  park_rows(0, TM);
 #pragma unroll
   for (int r = 0; r < WM; r += kRowsPerPass) {
     const int row = r + erow;
