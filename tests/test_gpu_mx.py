@@ -469,6 +469,32 @@ def test_mx_gemm_small_vs_c_oracle_exact_products(d):
     assert torch.equal(out.cpu(), ref.bfloat16())
 
 
+@pytest.mark.parametrize("size", [(16, 256, 136), (40, 352, 264), (64, 1152, 48)], ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+@pytest.mark.parametrize("tiles", [1, 2])
+def test_mx_gemm_few_rows_kernel_vs_c_oracle_exact_products(d, cabi, size, tiles):
+    """the kernel for few rows on operands whose products and partial sums are exact (see the test above):
+    bit for bit the C oracle's float64 reference rounded to bf16, for one and two 16-column tiles per
+    wave and a K with a partly filled last step"""
+    M, K, N = size
+    g = util.gen(84 + M)
+    a = torch.exp2(torch.randint(-3, 3, (M, K), generator=g).float()) * torch.where(torch.rand(M, K, generator=g) < 0.5, -1.0, 1.0)
+    b = torch.exp2(torch.randint(-3, 3, (N, K), generator=g).float()) * torch.where(torch.rand(N, K, generator=g) < 0.5, -1.0, 1.0)
+    a = a * (torch.rand(M, K, generator=g) < 0.02)
+    b = b * (torch.rand(N, K, generator=g) < 0.5)
+    ad, asc = d.mx_fp8_quantize(a.bfloat16().cuda())
+    bd, bsc = d.mx_fp8_quantize(b.bfloat16().cuda())
+    cabi.set_tuning("gemm.variant", 9)
+    cabi.set_tuning("gemm.few_rows_tiles", tiles)
+    try:
+        out = d.mx_fp8_bf16(ad, bd.t(), d.to_blocked(asc.view(M, K // 32)), d.to_blocked(bsc.view(N, K // 32)))
+    finally:
+        cabi.set_tuning("gemm.variant", 0)
+        cabi.set_tuning("gemm.few_rows_tiles", 0)
+    ref = co.mx_gemm_ref(util.codes(ad), util.codes(bd), co.to_blocked(util.codes(asc).view(M, K // 32)),
+                         co.to_blocked(util.codes(bsc).view(N, K // 32)))
+    assert torch.equal(out.cpu(), ref.bfloat16())
+
+
 def test_mx_gemm_scale_bytes_are_applied_per_row_and_kblock(d):
     M, K, N = 256, 512, 256
     a_data, a_sc, b_data, b_sc = _operands(d, M, K, N, 83, "randn")

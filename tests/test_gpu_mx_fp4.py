@@ -147,6 +147,30 @@ def test_mx_fp4_gemm_bit_exact_when_sums_fit_fp32(d):
         assert torch.equal(out.cpu(), ref.bfloat16())
 
 
+@pytest.mark.parametrize("tiles", [1, 2])
+def test_mx_fp4_gemm_few_rows_kernel_bit_exact_when_sums_fit_fp32(d, cabi, tiles):
+    """the kernel for few rows on the operands of the test above (exact in fp32 in any order): bit for bit
+    the C oracle's reference, for one and two 16-column tiles per wave, every count of 16-row tiles and a K
+    with a partly filled last 128-element step"""
+    g = util.gen(92)
+    cabi.set_tuning("gemm.variant", 9)
+    cabi.set_tuning("gemm.few_rows_tiles", tiles)
+    try:
+        for (M, K, N) in ((16, 384, 136), (33, 480, 264), (64, 1312, 48), (50, 512, 40)):
+            a = torch.randint(0, 16, (M, K), generator=g, dtype=torch.uint8) * (torch.rand(M, K, generator=g) < 0.03)
+            b = torch.randint(0, 16, (N, K), generator=g, dtype=torch.uint8) * (torch.rand(N, K, generator=g) < 0.5)
+            ap = (a[:, 0::2] | (a[:, 1::2] << 4)).to(torch.uint8)
+            bp = (b[:, 0::2] | (b[:, 1::2] << 4)).to(torch.uint8)
+            sa = torch.randint(125, 130, (M, K // 32), generator=g, dtype=torch.uint8)
+            sb = torch.randint(125, 130, (N, K // 32), generator=g, dtype=torch.uint8)
+            out = _run(d, ap, sa, bp, sb)
+            ref = co.mx_fp4_gemm_ref(ap, bp, co.to_blocked(sa), co.to_blocked(sb))
+            assert torch.equal(out.cpu(), ref.bfloat16()), (M, K, N)
+    finally:
+        cabi.set_tuning("gemm.variant", 0)
+        cabi.set_tuning("gemm.few_rows_tiles", 0)
+
+
 def test_mx_fp4_gemm_scales_per_row_and_kblock(d):
     M, K, N = 256, 640, 256
     a, sa, b, sb = _operands(M, K, N, 93, "randn")
