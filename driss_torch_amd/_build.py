@@ -6,7 +6,9 @@
   only, linked against torch and the kernel library.
 
 Run ``python driss_torch_amd/_build.py`` (or ``__graft_entry__.build()``).  The GPU is not
-needed: hipcc cross-compiles.
+needed: hipcc cross-compiles.  ``python driss_torch_amd/_build.py --phase-log`` makes a third library,
+``lib/libdriss_torch_hip_phases.so``: the kernels with their per-workgroup clock readings compiled in,
+which only ``bench.py --phases`` loads.
 """
 from __future__ import annotations
 
@@ -26,6 +28,7 @@ ROCM = Path(os.environ.get("ROCM_PATH", "/opt/rocm"))
 
 HIP_LIB = LIB / "libdriss_torch_hip.so"
 TORCH_LIB = LIB / "libdriss_torch.so"
+PHASES_HIP_LIB = LIB / "libdriss_torch_hip_phases.so"  # made on request only (--phase-log)
 
 HIP_SOURCES = ["abi_common.hip", "amax.hip", "saturated_cast.hip", "dynamic_scaled_quant.hip", "mx_cast.hip",
                "mx_fp8_bf16.hip"]
@@ -50,21 +53,26 @@ def _run(cmd: list[str]) -> None:
         sys.stderr.write("\n".join(noise) + "\n")
 
 
-def build_hip_library(jobs: int = 6) -> Path:
-    OBJ.mkdir(parents=True, exist_ok=True)
+def build_hip_library(jobs: int = 6, phase_log: bool = False) -> Path:
+    """The kernel library; with ``phase_log`` the instrumented build of the same sources
+    (-DDT_PHASE_LOG: per-workgroup clock readings and dt_set_phase_log, for ``bench.py --phases``)."""
+    obj_dir = OBJ / "phases" if phase_log else OBJ
+    target = PHASES_HIP_LIB if phase_log else HIP_LIB
+    obj_dir.mkdir(parents=True, exist_ok=True)
     hipcc = str(ROCM / "bin" / "hipcc")
+    flags = HIPCC_FLAGS + (["-DDT_PHASE_LOG"] if phase_log else [])
     objs = []
 
     def compile_one(src: str) -> str:
-        obj = OBJ / (Path(src).stem + ".o")
-        _run([hipcc, *HIPCC_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", "-c", str(CSRC / src), "-o", str(obj)])
+        obj = obj_dir / (Path(src).stem + ".o")
+        _run([hipcc, *flags, f"-I{INCLUDE}", f"-I{CSRC}", "-c", str(CSRC / src), "-o", str(obj)])
         return str(obj)
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = list(pool.map(compile_one, HIP_SOURCES))
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wno-unused-command-line-argument", *objs, "-o",
-          str(HIP_LIB)])
-    return HIP_LIB
+          str(target)])
+    return target
 
 
 def build_torch_shim() -> Path:
@@ -90,5 +98,8 @@ def build_all() -> None:
 
 
 if __name__ == "__main__":
-    build_all()
-    print("built", HIP_LIB, TORCH_LIB)
+    if "--phase-log" in sys.argv[1:]:
+        print("built", build_hip_library(phase_log=True))
+    else:
+        build_all()
+        print("built", HIP_LIB, TORCH_LIB)

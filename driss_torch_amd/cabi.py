@@ -12,6 +12,9 @@ from pathlib import Path
 import torch
 
 _LIB_PATH = Path(__file__).parent / "lib" / "libdriss_torch_hip.so"
+# the same kernels built with -DDT_PHASE_LOG (python driss_torch_amd/_build.py --phase-log): per-workgroup
+# clock readings for the benchmark's phase report, switched on with dt_set_phase_log
+_PHASES_LIB_PATH = Path(__file__).parent / "lib" / "libdriss_torch_hip_phases.so"
 
 OK = 0
 F32, BF16, F16 = 0, 1, 2
@@ -49,7 +52,9 @@ SIGNATURES = {
     "dt_mx_fp8_bf16_ws": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "dt_mx_fp4_bf16_ws": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "dt_dynamic_quant_gave_up": (_i32, []),
-    "dt_set_phase_log": (_i32, [_vp, _sz]),
+    "dt_set_exclusive_gpu": (_i32, [_i32]),
+    "dt_get_exclusive_gpu": (_i32, []),
+    "dt_dynamic_quant_resident_launches": (C.c_uint64, []),
     "dt_set_tuning": (_i32, [_cp, _i32]),
     "dt_get_tuning": (_i32, [_cp, C.POINTER(_i32)]),
 }
@@ -57,18 +62,35 @@ SIGNATURES = {
 _lib = None
 
 
+def _load(path: Path, extra=None) -> C.CDLL:
+    if not path.exists():
+        raise ImportError(f"{path} is missing: build it with `python driss_torch_amd/_build.py`")
+    L = C.CDLL(str(path))
+    for name, (res, args) in {**SIGNATURES, **(extra or {})}.items():
+        fn = getattr(L, name)
+        fn.restype, fn.argtypes = res, args
+    return L
+
+
 def lib() -> C.CDLL:
     """The kernel library.  Raises if it has not been built -- there is no fallback."""
     global _lib
     if _lib is None:
-        if not _LIB_PATH.exists():
-            raise ImportError(f"{_LIB_PATH} is missing: build it with `python driss_torch_amd/_build.py`")
-        L = C.CDLL(str(_LIB_PATH))
-        for name, (res, args) in SIGNATURES.items():
-            fn = getattr(L, name)
-            fn.restype, fn.argtypes = res, args
-        _lib = L
+        _lib = _load(_LIB_PATH)
     return _lib
+
+
+def use_phase_log_build() -> C.CDLL:
+    """Switch this module's wrappers to the instrumented build of the kernels (benchmark only)."""
+    global _lib
+    _lib = _load(_PHASES_LIB_PATH, {"dt_set_phase_log": (_i32, [_vp, _sz])})
+    return _lib
+
+
+def set_exclusive_gpu(on: bool) -> None:
+    """Say that this process has the GPU to itself (or no longer): per-tensor dynamic quantization of a
+    tensor that fits the chip then runs as one kernel that waits inside for all of its workgroups."""
+    _check(lib().dt_set_exclusive_gpu(1 if on else 0), "dt_set_exclusive_gpu")
 
 
 class DtError(RuntimeError):

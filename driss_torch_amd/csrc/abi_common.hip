@@ -1,5 +1,7 @@
 // Status strings, device facts, tuning knobs and the workspace entry points of the C ABI.
+#include <stdlib.h>
 #include <string.h>
+#include <strings.h>
 
 #include <atomic>
 #include <mutex>
@@ -16,7 +18,10 @@ struct Knob {
 };
 // Launch-shape knobs.  Workgroups per CU for the persistent grids, chosen on MI355X.
 //   dynamic.resident: 1 = per-tensor dynamic quantization of a tensor that fits the chip runs as one
-//                 kernel that keeps it in registers and LDS; dynamic.resident_min_kib = smallest such
+//                 kernel that keeps it in registers and LDS.  That kernel waits inside for all of its
+//                 workgroups and so assumes that this process has the GPU to itself: 0 unless the caller
+//                 opts in (dt_set_exclusive_gpu, or DRISS_TORCH_RESIDENT=1 in the environment when the
+//                 library is loaded); dynamic.resident_min_kib = smallest such
 //                 tensor; sizes in [resident_gap_lo_kib, resident_gap_hi_kib) take the two kernels
 //                 dynamic.resident_overflow: 1 = tensors of up to 4 x the chip's capacity keep what fits
 //                 and read only the rest twice
@@ -55,7 +60,7 @@ Knob g_knobs[] = {
     {"gemm.variant", 0},
     {"gemm.split_k", 0},
     {"gemm.tail_quads", 1},
-    {"dynamic.resident", 1},
+    {"dynamic.resident", 0},
     {"dynamic.resident_min_kib", 32768},
     {"dynamic.resident_gap_lo_kib", 0},
     {"dynamic.resident_gap_hi_kib", 0},
@@ -64,8 +69,27 @@ Knob g_knobs[] = {
 };
 constexpr int kNumKnobs = sizeof(g_knobs) / sizeof(g_knobs[0]);
 
+// DRISS_TORCH_RESIDENT: "1", "on", "true", "yes" (any case) switch the one-kernel dynamic quantization on;
+// anything else, or no variable, leaves it off.
+bool resident_opt_in_from(const char* v) {
+  if (!v) return false;
+  for (const char* yes : {"1", "on", "true", "yes"})
+    if (strcasecmp(v, yes) == 0) return true;
+  return false;
+}
+struct KnobsFromEnvironment {
+  KnobsFromEnvironment() {
+    if (resident_opt_in_from(getenv("DRISS_TORCH_RESIDENT")))
+      for (int i = 0; i < kNumKnobs; ++i)
+        if (strcmp(g_knobs[i].key, "dynamic.resident") == 0) g_knobs[i].value.store(1, std::memory_order_relaxed);
+  }
+} g_knobs_from_environment;  // after g_knobs in this file: initialised after it, when the library is loaded
+
+#ifdef DT_PHASE_LOG
 std::atomic<uint64_t*> g_phase_log{nullptr};
 std::atomic<size_t> g_phase_log_bytes{0};
+std::atomic<int> g_phase_log_device{-1};
+#endif
 
 constexpr int kMaxDevices = 16;
 DeviceFacts g_facts[kMaxDevices];
@@ -78,10 +102,15 @@ int tuning(const char* key) {
   return 0;
 }
 
+#ifdef DT_PHASE_LOG
 uint64_t* phase_log(size_t need_bytes) {
   uint64_t* p = g_phase_log.load(std::memory_order_relaxed);
-  return p && g_phase_log_bytes.load(std::memory_order_relaxed) >= need_bytes ? p : nullptr;
+  if (!p || g_phase_log_bytes.load(std::memory_order_relaxed) < need_bytes) return nullptr;
+  int dev = -1;
+  (void)hipGetDevice(&dev);
+  return dev == g_phase_log_device.load(std::memory_order_relaxed) ? p : nullptr;  // the buffer's own device only
 }
+#endif
 
 const DeviceFacts& device_facts() {
   int dev = 0;
@@ -136,12 +165,18 @@ int dt_workspace_init(void* workspace, size_t workspace_bytes, dt_stream_t strea
   return dt::launch_status();
 }
 
+#ifdef DT_PHASE_LOG
 int dt_set_phase_log(void* device_buffer, size_t bytes) {
   if (device_buffer && !dt::aligned(device_buffer, 8)) return DT_ERR_MISALIGNED;
+  int dev = -1;
+  (void)hipGetDevice(&dev);
+  dt::g_phase_log.store(nullptr, std::memory_order_relaxed);
   dt::g_phase_log_bytes.store(device_buffer ? bytes : 0, std::memory_order_relaxed);
+  dt::g_phase_log_device.store(device_buffer ? dev : -1, std::memory_order_relaxed);
   dt::g_phase_log.store(static_cast<uint64_t*>(device_buffer), std::memory_order_relaxed);
   return DT_OK;
 }
+#endif
 
 int dt_set_tuning(const char* key, int value) {
   if (!key) return DT_ERR_NULL_POINTER;

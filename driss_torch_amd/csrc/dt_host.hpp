@@ -24,9 +24,18 @@ const DeviceFacts& device_facts();  // of the current device, cached per device
 
 int tuning(const char* key);  // current value of a launch knob
 
-// Device buffer for per-workgroup clock readings (dt_set_phase_log), or null when none is set or it
-// holds fewer than `need_bytes`.
+// Per-workgroup clock readings for the benchmark's phase report exist only in a build with
+// -DDT_PHASE_LOG (a second library made for that report); in the product build kPhaseLog is false, the
+// kernels' stamps compile to nothing and the entry point that sets the buffer is not there.
+#ifdef DT_PHASE_LOG
+constexpr bool kPhaseLog = true;
+// Device buffer for the readings (dt_set_phase_log), or null when none is set, it holds fewer than
+// `need_bytes`, or it lives on another device than the current one.
 uint64_t* phase_log(size_t need_bytes);
+#else
+constexpr bool kPhaseLog = false;
+inline uint64_t* phase_log(size_t) { return nullptr; }
+#endif
 
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 inline int64_t ceil_div(int64_t a, int64_t b) { return a / b + (a % b != 0); }  // src/include/utils.h:37-39

@@ -1,6 +1,7 @@
 // dt_dynamic_scaled_quant*: amax -> scale -> saturating fp8 cast, per tensor and per row (C ABI).
 //
-// A tensor that fits the chip's registers and LDS (128 MiB on 256 CUs) goes through one kernel
+// For a caller that has said that its process owns the GPU (dt_set_exclusive_gpu, DRISS_TORCH_RESIDENT=1),
+// a tensor that fits the chip's registers and LDS (128 MiB on 256 CUs) goes through one kernel
 // that holds it there between the reduction and the cast (resident_kernels.hpp).  Otherwise
 // the work is two stream-ordered kernels: the amax reduction, whose last workgroup also derives
 // the scale(s) into the workspace, and the streaming cast, which reads the scale from there;
@@ -139,3 +140,25 @@ extern "C" int dt_dynamic_scaled_quant_rowwise(const void* x, int in_dtype, int6
 }
 
 extern "C" int dt_dynamic_quant_gave_up(void) { return dt::resident_take_gave_up() ? 1 : 0; }
+
+extern "C" int dt_set_exclusive_gpu(int on) {
+  if (on) {
+    // the current device's word of pinned host memory now, so that no quantization call has to make it
+    // (a process without a usable device may still set the flag: the first launch tries again)
+    int dev = -1;
+    if (hipGetDevice(&dev) == hipSuccess) {
+      dt::ResidentGate& gate = dt::resident_gate();
+      std::lock_guard<std::mutex> lock(gate.mu);
+      (void)dt::resident_host_word_locked(gate, dev);
+    } else {
+      (void)hipGetLastError();
+    }
+  }
+  return dt_set_tuning("dynamic.resident", on ? 1 : 0);
+}
+
+extern "C" int dt_get_exclusive_gpu(void) { return dt::tuning("dynamic.resident") ? 1 : 0; }
+
+extern "C" uint64_t dt_dynamic_quant_resident_launches(void) {
+  return dt::resident_gate().launches.load(std::memory_order_relaxed);
+}

@@ -72,10 +72,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     int64_t ldo, int tiles_m, int tiles_n, int wide_stores, int splits, v4f* __restrict__ partial,
     uint32_t* __restrict__ tickets, int first_block, uint64_t* __restrict__ phase_log) {
   constexpr bool SPLIT = MODE == kSplitK;
-  // phase_log (normally null; dt_set_phase_log): per workgroup four readings of the 100 MHz constant-rate
-  // counter -- start, K loop entered, K loop left, output stored -- and where it ran (XCC_ID, HW_ID).
-  // The readings are taken always (three scalar reads per tile) and stored at the very end.
-  const uint64_t t_start = wall_clock64();
+  // phase_log (only in a build with DT_PHASE_LOG, and normally null there; dt_set_phase_log): per workgroup
+  // four readings of the 100 MHz constant-rate counter -- start, K loop entered, K loop left, output
+  // stored -- and where it ran (XCC_ID, HW_ID), stored at the very end.
+  auto clock_reading = []() -> uint64_t {
+    if constexpr (kPhaseLog) return wall_clock64();
+    else return 0;
+  };
+  const uint64_t t_start = clock_reading();
   static_assert(!(SPLIT && TOUCH), "the prefetch shares assume that a workgroup walks the whole K");
   static_assert(MODE != kQuads || (BM == 128 && BN == 128), "quadrants of a 256 x 256 tile");
   static_assert(MODE != kHalves || (BM == 256 && BN == 128), "halves of a 256 x 256 tile");
@@ -132,9 +136,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // K counts elements (a multiple of 32, the MX block); a row holds k_bytes bytes, a K-step is 128 of
   // them.  The last step may be partly filled.  Its loads then stay inside the row: a 16-byte chunk past
   // the end reads a valid chunk of the same row again (tail_adj), and what it reads does not count,
-  // because its K-blocks are the zero padding of the blocked scale buffers: byte 0 on both sides scales
-  // the block's sum by 2^-254, which leaves the accumulator as it is (the re-read payload is finite
-  // unless the row holds a NaN, and then the row's results are NaN anyway).  With FP4 a step is two
+  // because the scale bytes of its K-blocks are zero: byte 0 on both sides scales the block's sum by
+  // 2^-254, which leaves the accumulator as it is (the re-read payload is finite unless the row holds
+  // a NaN, and then the row's results are NaN anyway).  Those bytes are the padding of the caller's
+  // blocked scale buffers, which nobody can check: whatever they hold, the staged copy of the partly
+  // filled step's scale chunks is overwritten with zeros there before anybody reads it
+  // (mask_tail_scales).  With FP4 a step is two
   // 128-element scale chunks; when the last step has no second chunk at all (K % 256 in 1..128) its
   // second MFMA is switched off through the scale operand (see scale_bits).
   const int k_bytes = FP4 ? K / 2 : K;
@@ -294,6 +301,24 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   };
   auto touch = [&](int step) { touch_at(touch_address(step)); };
 
+  // The staged scale chunks of the partly filled step, once they have landed in ring slot `stage`: a
+  // word holds the four K-block bytes of a row; the bytes of K-blocks past the end of K become 0.  A
+  // slot is 256 words per operand and chunk, one per thread; the caller puts a barrier behind this.
+  static_assert(kWaves * kWave * 4 == 1024, "one scale word per thread and 1 KiB slot");
+  const int k_blocks = K / 32;
+  auto mask_tail_scales = [&](uint32_t stage) {
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const int valid = k_blocks - ((ks_begin + tail_step) * KC + c) * 4;  // K-blocks of this chunk inside K
+      if (valid >= 4) continue;
+      const uint32_t keep = valid <= 0 ? 0u : (1u << (8 * valid)) - 1u;
+      uint32_t* const wa = reinterpret_cast<uint32_t*>(lds + stage + kOffSA + c * 1024) + tid;
+      uint32_t* const wb = reinterpret_cast<uint32_t*>(lds + stage + kOffSB + c * 1024) + tid;
+      *wa &= keep;
+      *wb &= keep;
+    }
+  };
+
   v4f acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -401,6 +426,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   for (int p = 0; p < kTouchAhead; ++p) touch(NST + p);
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 1) * kLoadsPerStep + kTouchAhead * kTouch) : "memory");
   __syncthreads();
+  if (tail_step == 0) {  // a single, partly filled step: its scales are read next
+    mask_tail_scales(0u);
+    __syncthreads();
+  }
   const int a_row0 = wm * WM, b_row0 = wn * WN;
   // only the wave's first row differs between waves: fold it into the per-lane bases
   const uint32_t lane_lo_a = frag_lo + (a_row0 >> 3) * kGroupStride, lane_hi_a = frag_hi + (a_row0 >> 3) * kGroupStride;
@@ -428,7 +457,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
 
   // every refill of the loop is the partly filled step (the loop clamps a refill at the last step)
   if (tail_step >= 0 && tail_step < NST) tail_in_place();
-  const uint64_t t_loop = wall_clock64();
+  const uint64_t t_loop = clock_reading();
   // What a step needs of its ring slot `cur` and of the next step's `nxt`: the slots' offsets and the
   // per-lane fragment and scale addresses in them.  They are carried from step to step (this step's
   // `nxt` set is the next step's `cur` set) and the new `nxt` set is worked out in the middle of the
@@ -535,6 +564,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
     // touch has to stay the youngest: it misses the L2 by design, and loads complete in order)
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_waitcnt vmcnt(%0)" ::"n"((NST - 2) * kVmPerStep + kTouch) : "memory");
     __syncthreads();
+    if (ks + 1 == tail_step) {  // the partly filled last step has landed: nobody has read its scales yet
+      mask_tail_scales(nxt);
+      __syncthreads();
+    }
     __builtin_amdgcn_sched_barrier(0);
     // ---- behind the bar: (hi,hi) reloads a[lo], (hi,lo) reloads b[hi], both from step ks+1
     constexpr int kFirstFrag = HA > 2 ? 1 : 0;  // a[lo] fragments at kFirstFrag + k * kFragEvery, DMA loads in between
@@ -585,7 +618,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
   // (the no-ops cover the distance an assembly-written MFMA needs before its result is read)
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  const uint64_t t_loop_end = wall_clock64();
+  const uint64_t t_loop_end = clock_reading();
 
   if constexpr (SPLIT) {
     __shared__ uint32_t drawn;
@@ -700,7 +733,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void mx_gemm_kernel(
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (phase_log) {
+    if (kPhaseLog && phase_log) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       if (threadIdx.x == 0) {
         uint64_t* const e = phase_log + (size_t)blockIdx.x * 8;

@@ -61,10 +61,13 @@ __global__ __launch_bounds__(kBlock) void amax_kernel(const void* __restrict__ x
   constexpr int kB = InTraits<IN>::kBytes, kV = InTraits<IN>::kVec;
   __shared__ uint32_t lds[kBlock / kWave];
   const int tid = threadIdx.x;
-  // phase_log (normally null): readings of the constant-rate 100 MHz counter per workgroup -- start,
-  // share loaded, workgroup's maximum known, atomics done -- for the benchmark's per-phase report
+  // phase_log (only in a build with DT_PHASE_LOG, and normally null there): readings of the constant-rate
+  // 100 MHz counter per workgroup -- start, share loaded, workgroup's maximum known, atomics done -- for
+  // the benchmark's per-phase report
   auto stamp = [&](int k) {
-    if (phase_log && tid == 0) phase_log[blockIdx.x * 4 + k] = wall_clock64();
+    if constexpr (kPhaseLog) {
+      if (phase_log && tid == 0) phase_log[blockIdx.x * 4 + k] = wall_clock64();
+    }
   };
   stamp(0);
   const u32x4* v = reinterpret_cast<const u32x4*>(static_cast<const uint8_t*>(x) + sp.head * kB);

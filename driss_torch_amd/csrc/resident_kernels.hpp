@@ -99,11 +99,13 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
   const u32x4* v = static_cast<const u32x4*>(x);
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   const int64_t first = (int64_t)blockIdx.x * kBlock + tid;
-  // phase_log (normally null): four readings of the constant-rate 100 MHz counter per workgroup --
+  // phase_log (only in a build with DT_PHASE_LOG, and normally null there): four readings of the constant-rate 100 MHz counter per workgroup --
   // start, share loaded and reduced, released from the grid barrier, done -- for the benchmark's
   // per-phase report.  The counter is common to all CUs, so readings of different workgroups compare.
   auto stamp = [&](int k) {
-    if (phase_log && tid == 0) phase_log[blockIdx.x * 4 + k] = wall_clock64();
+    if constexpr (kPhaseLog) {
+      if (phase_log && tid == 0) phase_log[blockIdx.x * 4 + k] = wall_clock64();
+    }
   };
   stamp(0);
 
@@ -236,6 +238,7 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
   uint32_t* depart = reinterpret_cast<uint32_t*>(ws + kWsDepart);
   // (1 << 32) | amax bits once everybody has arrived; this workgroup polls its own copy
   uint64_t* release = reinterpret_cast<uint64_t*>(ws + kWsRelease + (blockIdx.x % kWsReleaseWords) * kWsReleaseStep);
+  bool gave_up_here = false;  // thread 0's: this workgroup stopped waiting
   if (tid == 0) {
     uint32_t before = __hip_atomic_fetch_max(running, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     uint32_t one = 1u;  // the ticket depends on the returned value, so the two atomics stay ordered
@@ -260,6 +263,7 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
           // and tell the host (a word of pinned host memory): the library's next call on this device reports it
           if (host_flag) __hip_atomic_store(host_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
           rel = 0x7FC00000ull;  // the outputs of this workgroup become NaN: a loud failure
+          gave_up_here = true;
           break;
         }
       }
@@ -355,10 +359,12 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
     out[e] = cast_one<IN, OUT, ROUND_BF16>(x, e, s);
     if constexpr (PAIR) out2[e] = cast_one<IN, OUT2, ROUND_BF16>(x, e, s2);
   }
-  if (phase_log) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores of this wave have left
-    __syncthreads();
-    stamp(3);
+  if constexpr (kPhaseLog) {
+    if (phase_log) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores of this wave have left
+      __syncthreads();
+      stamp(3);
+    }
   }
   // ---- departure, at the very end: counted here and not at the barrier, where the atomic's round trip
   // (the 256 of them queue on one address) held every workgroup back by 1.5-3 us before its stores.  The
@@ -367,7 +373,11 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
     // everything this wave has sent to memory has been performed, the release words of the last
     // arriver included: whoever finds itself last may put them back to zero
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (__hip_atomic_fetch_add(depart, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1) {
+    // the counter's low half counts departures, its high half those of workgroups that gave up: the last
+    // one to leave then knows whether any part of the output is NaN without another round trip
+    const uint32_t left_before = __hip_atomic_fetch_add(depart, gave_up_here ? 0x10001u : 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((left_before & 0xFFFFu) == gridDim.x - 1) {
+      const bool any_gave_up = gave_up_here || (left_before >> 16) != 0;
       __hip_atomic_store(running, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(depart, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -375,7 +385,8 @@ __global__ __launch_bounds__(kBlock) void resident_quant_kernel(const void* __re
       for (uint32_t j = 0; j < kWsReleaseWords; ++j)
         __hip_atomic_store(reinterpret_cast<uint64_t*>(ws + kWsRelease + j * kWsReleaseStep), 0ull, __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
-      const float amax_final = as_f32(bcast);
+      // after a give-up anywhere amax and the scales are NaN like the outputs of the workgroups that gave up
+      const float amax_final = any_gave_up ? as_f32(0x7FC00000u) : as_f32(bcast);
       float* wscale = reinterpret_cast<float*>(ws + kWsScale);
       *reinterpret_cast<float*>(ws + kWsAmax) = amax_final;
       if (amax_out) *amax_out = amax_final;
@@ -403,10 +414,28 @@ struct ResidentGate {
   // next per-tensor dynamic quantization on that device.
   volatile uint32_t* gave_up_host[kMaxDevices] = {};
   uint32_t* gave_up_dev[kMaxDevices] = {};
+  std::atomic<uint64_t> launches{0};  // one-kernel launches of this process (dt_dynamic_quant_resident_launches)
 };
 inline ResidentGate& resident_gate() {
   static ResidentGate* g = new ResidentGate();  // leaked on purpose: no HIP calls at process exit
   return *g;
+}
+
+// The device's word of pinned host memory, made if it is not there yet (gate.mu held).  False when it
+// cannot be made.  dt_set_exclusive_gpu(1) calls this up front so that no quantization call allocates.
+inline bool resident_host_word_locked(ResidentGate& gate, int dev) {
+  if (dev < 0 || dev >= ResidentGate::kMaxDevices) return false;
+  if (gate.gave_up_host[dev]) return true;
+  void* host = nullptr;
+  void* devp = nullptr;
+  if (hipHostMalloc(&host, 64, hipHostMallocMapped) != hipSuccess || hipHostGetDevicePointer(&devp, host, 0) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  *static_cast<volatile uint32_t*>(host) = 0u;
+  gate.gave_up_host[dev] = static_cast<volatile uint32_t*>(host);
+  gate.gave_up_dev[dev] = static_cast<uint32_t*>(devp);
+  return true;
 }
 
 // True when the process runs under a CU mask given through the environment, which
@@ -505,17 +534,7 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
   // every workgroup waits for all the others: a stream that may not use as many CUs as the grid has
   // workgroups could never hold them all at once
   if (stream_cu_count(stream) < grid || cu_mask_in_environment()) return kResidentNotTaken;
-  if (!gate.gave_up_host[dev]) {
-    void* host = nullptr;
-    void* devp = nullptr;
-    if (hipHostMalloc(&host, 64, hipHostMallocMapped) != hipSuccess || hipHostGetDevicePointer(&devp, host, 0) != hipSuccess) {
-      (void)hipGetLastError();
-      return kResidentNotTaken;  // without a way to report a give-up the path is not taken
-    }
-    *static_cast<volatile uint32_t*>(host) = 0u;
-    gate.gave_up_host[dev] = static_cast<volatile uint32_t*>(host);
-    gate.gave_up_dev[dev] = static_cast<uint32_t*>(devp);
-  }
+  if (!resident_host_word_locked(gate, dev)) return kResidentNotTaken;  // without a way to report a give-up the path is not taken
   uint64_t* const log = phase_log((size_t)grid * 32);
   if (gate.used[dev] && gate.last_stream[dev] != stream) {
     // mark the tail of the stream that ran the previous resident kernel and wait for it here
@@ -538,6 +557,7 @@ inline int launch_resident_impl(const void* x, int64_t numel, void* ws, void* ou
   if (st == DT_OK) {
     gate.used[dev] = true;
     gate.last_stream[dev] = stream;
+    gate.launches.fetch_add(1, std::memory_order_relaxed);
   }
   return st;
   }

@@ -4,9 +4,11 @@
  * Plain pointers and sizes only: no torch types, no C++ types, no exceptions.  Every entry
  * point validates its arguments on the host, enqueues its kernels on `stream` (NULL = the
  * legacy default stream), never synchronises, never allocates device memory, and returns a
- * dt_status code.  (One exception to "never allocates": the first per-tensor dynamic quantization
- * that takes the one-kernel path on a device makes one 64-byte block of pinned HOST memory and keeps
- * it, see dt_dynamic_scaled_quant.)  All data pointers are device pointers on the current HIP device.
+ * dt_status code.  (One exception to "never allocates", for callers that opted in with
+ * dt_set_exclusive_gpu / DRISS_TORCH_RESIDENT only: the one-kernel path of the per-tensor dynamic
+ * quantization keeps one 64-byte block of pinned HOST memory per device, made by dt_set_exclusive_gpu(1)
+ * or at the first such launch, see dt_dynamic_scaled_quant.)  All data pointers are device pointers on
+ * the current HIP device.
  *
  * Each declaration cites the reference (drisspg/driss_torch) interface it stands in for;
  * paths are relative to the reference tree.  The torch-facing registration shim
@@ -105,7 +107,7 @@ DT_API int dt_saturated_cast(const void* x, int in_dtype, int64_t numel, const f
  * own `fmax / (amax + 1e-12)` at :111 differs in the last bits).  amax_out / scale_out may
  * be NULL.  The reference runs fp32 input only (:130,135); bf16 is accepted here.
  *
- * A tensor that fits the chip (128 MiB on 256 CUs, up to 4 x that partly) is quantized by ONE kernel
+ * With the opt-in below, a tensor that fits the chip (128 MiB on 256 CUs, up to 4 x that partly) is quantized by ONE kernel
  * that occupies every CU and waits inside for all of its workgroups, where the reference uses a
  * cooperative launch (:144-150).  That assumes THIS PROCESS OWNS THE GPU: the library chains such
  * launches of one process, and avoids streams with a CU mask, processes with a CU mask in the
@@ -114,10 +116,22 @@ DT_API int dt_saturated_cast(const void* x, int in_dtype, int64_t numel, const f
  * their outputs, amax and scale are NaN, every kernel still runs to its end, a word of pinned host
  * memory is set, and the NEXT dt_dynamic_scaled_quant / _pair call on that device launches nothing,
  * returns DT_ERR_RESIDENT_GAVE_UP once and switches the one-kernel path off for the process
- * (dt_set_tuning("dynamic.resident", 0); calls after that take the two kernels).  The workspace stays
+ * (calls after that take the two kernels).  The workspace stays
  * usable.  dt_dynamic_quant_gave_up() asks the same question without a quantization call: 1 if a
  * completed launch on the current device gave up since the last time it was asked (and clears it).
- * dt_set_tuning("dynamic.resident", 0) up front avoids the one-kernel path altogether.            */
+ *
+ * Because of that assumption the one-kernel path is OFF unless the caller opts in: dt_set_exclusive_gpu(1)
+ * (or DRISS_TORCH_RESIDENT=1 in the environment when the library is loaded; "0" or unset = off).  Without
+ * the opt-in every call runs the reduction kernel followed by the cast kernel, which wait for nothing and
+ * cannot produce NaN where the reference's cooperative launch could not.  dt_set_exclusive_gpu(1) also
+ * makes the current device's block of pinned host memory, so that no later call allocates; with the
+ * environment variable alone the first one-kernel launch on a device makes it.  The setting is one per
+ * process, not per device, and so is the switch-off after a give-up.  dt_get_exclusive_gpu() returns it;
+ * dt_dynamic_quant_resident_launches() counts the one-kernel launches of this process so far.
+ * The call that returns DT_ERR_RESIDENT_GAVE_UP wrote nothing to its outputs: repeat it.             */
+DT_API int dt_set_exclusive_gpu(int on);
+DT_API int dt_get_exclusive_gpu(void);
+DT_API uint64_t dt_dynamic_quant_resident_launches(void);
 DT_API int dt_dynamic_quant_gave_up(void);
 DT_API int dt_dynamic_scaled_quant(const void* x, int in_dtype, int64_t numel, int out_dtype,
                                    int round_mode, void* out, float* amax_out, float* scale_out,
@@ -277,12 +291,18 @@ DT_API int dt_mx_fp4_bf16_ws(const void* a, const void* b, const uint8_t* sfa, c
 DT_API int dt_set_tuning(const char* key, int value);
 DT_API int dt_get_tuning(const char* key, int* value);
 
-/* Benchmarking aid, no counterpart in the reference: while a device buffer is set here (8-byte aligned,
- * at least 32 bytes per workgroup of the kernel's grid; NULL switches it off), every one-kernel dynamic
- * quantization and every amax reduction writes four readings of the 100 MHz constant-rate counter
- * per workgroup into it (uint64[workgroup][4]: start; share loaded and reduced / loaded; released from
- * the grid barrier / workgroup maximum known; stores done / atomics done).                          */
+#ifdef DT_PHASE_LOG
+/* Benchmarking aid, no counterpart in the reference, and NOT part of the product library: it exists only
+ * in a second build of the kernels with -DDT_PHASE_LOG (python driss_torch_amd/_build.py --phase-log ->
+ * lib/libdriss_torch_hip_phases.so), which the benchmark loads for its per-phase report.  While a device
+ * buffer is set here (8-byte aligned, at least 32 bytes per workgroup of the kernel's grid, 64 for the
+ * GEMM; NULL switches it off), every one-kernel dynamic quantization, amax reduction and block-scaled GEMM
+ * launched on the buffer's device writes readings of the 100 MHz constant-rate counter per workgroup into
+ * it (uint64[workgroup][4]: start; share loaded and reduced / loaded; released from the grid barrier /
+ * workgroup maximum known; stores done / atomics done).  The buffer must outlive every such launch;
+ * launches on other devices ignore it.                                                              */
 DT_API int dt_set_phase_log(void* device_buffer, size_t bytes);
+#endif
 
 #ifdef __cplusplus
 }

@@ -13,7 +13,10 @@ HEADER = (ROOT / "include" / "driss_torch_hip.h").read_text()
 
 
 def _declared():
-    return sorted(set(re.findall(r"DT_API\s+[\w\s\*]+?\b(dt_\w+)\s*\(", HEADER)))
+    # what the product library must export: everything outside the DT_PHASE_LOG block (the benchmark's
+    # instrumented build, a library of its own)
+    product = re.sub(r"#ifdef DT_PHASE_LOG.*?#endif", "", HEADER, flags=re.S)
+    return sorted(set(re.findall(r"DT_API\s+[\w\s\*]+?\b(dt_\w+)\s*\(", product)))
 
 
 def test_library_exports_every_declared_symbol():
@@ -28,6 +31,47 @@ def test_library_exports_every_declared_symbol():
     assert L.dt_abi_version() == 1
     assert L.dt_status_string(0) == b"ok"
     assert L.dt_workspace_bytes() >= 4096
+    # the per-phase clock readings are not in the product: neither the entry point nor its declaration
+    assert "dt_set_phase_log" not in names and "dt_set_phase_log" in HEADER
+    with pytest.raises(AttributeError):
+        L.dt_set_phase_log
+
+
+@pytest.mark.parametrize("value,expect", [(None, 0), ("0", 0), ("1", 1), ("true", 1), ("ON", 1), ("Yes", 1), ("no", 0),
+                                          ("", 0), ("2", 0)])
+def test_one_kernel_dynamic_quant_is_opt_in(value, expect):
+    """the one-kernel per-tensor dynamic quantization assumes that the process owns the GPU: off unless
+    DRISS_TORCH_RESIDENT says otherwise when the library is loaded, or dt_set_exclusive_gpu is called
+    (a fresh process per case: the variable is read once, at load)"""
+    import os
+    import subprocess
+    import sys
+
+    from driss_torch_amd import cabi
+
+    env = {k: v for k, v in os.environ.items() if k != "DRISS_TORCH_RESIDENT"}
+    if value is not None:
+        env["DRISS_TORCH_RESIDENT"] = value
+    code = ("import ctypes as C, sys; L = C.CDLL(sys.argv[1]); v = C.c_int(-1); "
+            "assert L.dt_get_tuning(b'dynamic.resident', C.byref(v)) == 0; "
+            "print(v.value, L.dt_get_exclusive_gpu())")
+    out = subprocess.run([sys.executable, "-c", code, str(cabi._LIB_PATH)], env=env, capture_output=True, text=True, check=True)
+    assert out.stdout.split() == [str(expect), str(expect)]
+
+
+def test_exclusive_gpu_switch_without_gpu():
+    """dt_set_exclusive_gpu flips the setting also where no device is usable (the pinned word is then made
+    at the first launch); the launch counter starts at zero"""
+    from driss_torch_amd import cabi
+
+    L = cabi.lib()
+    keep = L.dt_get_exclusive_gpu()
+    try:
+        assert L.dt_set_exclusive_gpu(1) == 0 and L.dt_get_exclusive_gpu() == 1 and cabi.get_tuning("dynamic.resident") == 1
+        assert L.dt_set_exclusive_gpu(0) == 0 and L.dt_get_exclusive_gpu() == 0 and cabi.get_tuning("dynamic.resident") == 0
+        assert L.dt_dynamic_quant_resident_launches() >= 0
+    finally:
+        L.dt_set_exclusive_gpu(keep)
 
 
 def test_host_validation_without_gpu():

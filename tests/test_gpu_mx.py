@@ -255,6 +255,40 @@ def test_mx_gemm_k_of_any_whole_number_of_blocks(d, cabi, variant, K):
         cabi.set_tuning("gemm.variant", 0)
 
 
+def _poisoned_blocked(d, sc):
+    """the blocked layout of scale matrix `sc` [R, C] with every padding byte (rows past R, K-blocks past C)
+    set to 0xFF, the E8M0 NaN code, instead of zero"""
+    R, C = sc.shape
+    full = torch.full((-(-R // 128) * 128, -(-C // 4) * 4), 0xFF, dtype=torch.uint8, device=sc.device)
+    full[:R, :C] = sc.view(torch.uint8)
+    return d.to_blocked(full)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 7, 9])
+@pytest.mark.parametrize("size", [(40, 96, 264), (133, 160, 264), (64, 1120, 520), (300, 416, 136), (16, 4128, 2048)],
+                         ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+def test_mx_gemm_ignores_the_padding_of_the_scale_buffers(d, cabi, variant, size):
+    """the K-blocks past the end of K in a blocked scale buffer (K % 128 != 0) are padding that the caller may
+    have left uninitialised: with every padding byte set to the NaN code the result is the same bits as with
+    zeros, on every kernel (tiles of both sizes, shared K, few rows), for e4m3 and for e2m1 operands"""
+    M, K, N = size
+    if variant == 9 and M > 64:
+        pytest.skip("the kernel for few rows takes at most 64")
+    a_data, a_sc, b_data, b_sc = _operands(d, M, K, N, 4100 + K, "randn")
+    cabi.set_tuning("gemm.variant", variant)
+    try:
+        want = d.mx_fp8_bf16(a_data, b_data.t(), d.to_blocked(a_sc), d.to_blocked(b_sc))
+        got = d.mx_fp8_bf16(a_data, b_data.t(), _poisoned_blocked(d, a_sc), _poisoned_blocked(d, b_sc))
+        assert not got.isnan().any() and torch.equal(got, want)
+        # the same payload bytes read as e2m1 pairs: K/2 bytes hold K elements
+        a4, b4 = a_data.view(torch.uint8)[:, :K // 2].contiguous(), b_data.view(torch.uint8)[:, :K // 2].contiguous()
+        want4 = d.mx_fp4_bf16(a4, b4.t(), d.to_blocked(a_sc), d.to_blocked(b_sc))
+        got4 = d.mx_fp4_bf16(a4, b4.t(), _poisoned_blocked(d, a_sc), _poisoned_blocked(d, b_sc))
+        assert not got4.isnan().any() and torch.equal(got4, want4)
+    finally:
+        cabi.set_tuning("gemm.variant", 0)
+
+
 @pytest.mark.parametrize("size", [(1, 640, 8), (16, 2048, 256), (17, 96, 2056), (33, 1120, 264), (48, 416, 136), (64, 8192, 512),
                                   (5, 32, 24), (64, 160, 16)], ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
 def test_mx_gemm_few_rows_kernel(d, cabi, size):

@@ -221,6 +221,37 @@ def test_resident_not_taken_on_a_stream_restricted_to_some_cus(cabi):
     cabi.set_tuning("dynamic.resident_spin_limit", 1 << 19)
 
 
+def test_one_kernel_path_needs_the_opt_in(gpu_device):
+    """without the opt-in (dt_set_exclusive_gpu / DRISS_TORCH_RESIDENT) the torch op and the C ABI never
+    launch the kernel that waits for the whole chip, whatever the tensor's size: they run the reduction and
+    the cast, with the same bits; with it a tensor of 32 MiB and more takes the one kernel"""
+    import driss_torch_amd as d
+    from driss_torch_amd import cabi as c
+
+    L = c.lib()
+    keep = L.dt_get_exclusive_gpu()
+    x = util.normal_with_outliers((4096, 4096), 5)  # 32 MiB of bf16: the smallest size of the one-kernel path
+    xg = x.cuda()
+    ref, ramax, _ = co.dynamic_scaled_quant(x, E4, co.ROUND_V2)
+    try:
+        d.set_exclusive_gpu(False)
+        n0 = L.dt_dynamic_quant_resident_launches()
+        out = d.dynamic_scaled_quant(xg, E4)
+        o4, o5, amax, _ = d.dynamic_scaled_quant_pair(xg)
+        out_c, amax_c, _ = c.dynamic_scaled_quant(xg, E4, 2)
+        torch.cuda.synchronize()
+        assert L.dt_dynamic_quant_resident_launches() == n0
+        assert torch.equal(util.codes(out), ref) and torch.equal(util.codes(o4), ref) and torch.equal(util.codes(out_c), ref)
+        assert amax.item() == ramax.item() == amax_c.item()
+        d.set_exclusive_gpu(True)
+        out = d.dynamic_scaled_quant(xg, E4)
+        torch.cuda.synchronize()
+        assert L.dt_dynamic_quant_resident_launches() == n0 + 1
+        assert torch.equal(util.codes(out), ref)
+    finally:
+        L.dt_set_exclusive_gpu(keep)
+
+
 def test_resident_wait_gives_up_loudly(cabi):
     """with a spin limit of one poll most workgroups stop waiting before the last one has arrived:
     every wave still runs to the end, the sticky flag is set and those workgroups write NaN -- and
@@ -241,6 +272,8 @@ def test_resident_wait_gives_up_loudly(cabi):
         assert _timeout_flag(cabi) == 1
         codes = util.codes(out)
         assert ((codes & 0x7F) == 0x7F).any()
+        # amax and scale are NaN too, whichever workgroup was the last to leave
+        assert amax.isnan().all() and scale.isnan().all()
         cabi.set_tuning("dynamic.resident_spin_limit", 1 << 19)
         # the following call, through the torch op: an error, nothing launched, the path switched off
         with pytest.raises(RuntimeError, match="gave up"):
