@@ -30,8 +30,8 @@ HIP_LIB = LIB / "libdriss_torch_hip.so"
 TORCH_LIB = LIB / "libdriss_torch.so"
 PHASES_HIP_LIB = LIB / "libdriss_torch_hip_phases.so"  # made on request only (--phase-log)
 
-HIP_SOURCES = ["abi_common.hip", "amax.hip", "saturated_cast.hip", "dynamic_scaled_quant.hip", "mx_cast.hip",
-               "mx_fp8_bf16.hip"]
+HIP_SOURCES = ["mx_fp8_bf16.hip", "mx_few_rows.hip", "abi_common.hip", "amax.hip", "saturated_cast.hip",
+               "dynamic_scaled_quant.hip", "mx_cast.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-fno-fast-math",

@@ -45,10 +45,15 @@ struct Knob {
 //                 workspace of the _ws entry points), 1 = never, n = n workgroups per tile
 Knob g_knobs[] = {
     {"gemm.few_rows_tiles", 0},
+    {"gemm.few_rows_stagger", 1},
+    {"gemm.few_rows_waves", 0},
+    {"gemm.few_rows_steps", 0},
+    {"gemm.few_rows_per_cu", 0},
     {"amax.blocks_per_cu", 1},
     {"amax.stream_before_cast", 0},
-    {"cast.blocks_per_cu", 1},
-    {"cast.pair_blocks_per_cu", 1},
+    {"cast.blocks_per_cu", 0},
+    {"cast.unroll", 0},
+    {"cast.pair_blocks_per_cu", 0},
     {"rowwise.block_from_vecs", 257},
     {"mx.blocks_per_cu", 32},
     {"mx.col_blocks_per_cu", 32},

@@ -47,7 +47,7 @@ uint8_t* scratch_of_current_device(int* status) {
 }
 
 // the words a reduction expects to find zero (a fill kernel, not hipMemsetAsync: callers may capture)
-__global__ void clear_scratch_kernel(uint32_t* p) { p[threadIdx.x] = 0u; }
+__global__ void clear_scratch_kernel(uint32_t* p) { p[blockIdx.x * blockDim.x + threadIdx.x] = 0u; }
 }  // namespace
 
 extern "C" int dt_dynamic_scaled_quant(const void* x, int in_dtype, int64_t numel, int out_dtype, int round_mode,
@@ -79,7 +79,7 @@ extern "C" int dt_dynamic_scaled_quant_noalloc(const void* x, int in_dtype, int6
   hipStream_t s = dt::as_hip(stream);
   // The array keeps whatever the last call on this device left in it.  A completed call leaves its
   // counters at zero, but one that was cut short would not: start from zero every time.
-  clear_scratch_kernel<<<1, 128, 0, s>>>(reinterpret_cast<uint32_t*>(ws));
+  clear_scratch_kernel<<<dt::kWsBytes / 4 / 256, 256, 0, s>>>(reinterpret_cast<uint32_t*>(ws));
   if (int e = dt::launch_status()) return e;
   const float fm = fmax_of(out_dtype);
   st = in_dtype == DT_F32 ? dt::launch_amax<DT_F32>(x, numel, ws, amax_out, scale_out, 1, fm, 0.f, s)

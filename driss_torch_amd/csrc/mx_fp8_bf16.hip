@@ -24,6 +24,7 @@
 
 #include "dt_device.hpp"
 #include "dt_host.hpp"
+#include "mx_few_rows.hpp"
 
 namespace dt {
 
@@ -803,181 +804,6 @@ int launch_gemm(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const ui
   return launch_status();
 }
 
-// ---- few rows (M <= 64): the problem is the one pass over B, and a tile with a 128- or 256-row A
-// panel would idle most of its MFMAs and leave the chip to a handful of workgroups.  Here a workgroup
-// of 8 waves owns 16 rows of B (16 output columns) and every row of A; its waves share K between them
-// in turns of U K-steps, so the workgroup as a whole walks 16 whole rows of B front to back.  Nothing
-// goes through LDS on the way in: a lane's part of an MFMA operand is two 16-byte pieces of one row,
-// 64 bytes apart (one piece with e2m1), and the four lanes that share a row read 64 contiguous bytes
-// of it per load instruction (bytes 16 g .. of the step in lane group g); the E8M0 byte of a lane is one byte of the blocked scale buffer.  A's
-// rows come out of the L2 the same way (every workgroup reads all of A: M x K bytes, a few hundred
-// KiB).  A batch of U steps is in registers while the next one's loads are in flight.  The waves'
-// partial sums meet in LDS and are added in wave order; wave t writes the 16 x 16 tile of rows
-// 16 t .. 16 t + 15.  K-blocks past the end of K (K % 128 != 0) enter as zeros with a scale of 2^-127.
-template <bool FP4, int MT, int NT>
-__global__ __launch_bounds__(512) void mx_skinny_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
-                                                        const uint8_t* __restrict__ sfa, const uint8_t* __restrict__ sfb,
-                                                        int M, int N, int K, int64_t lda, int64_t ldb,
-                                                        uint16_t* __restrict__ out, int64_t ldo) {
-  constexpr int kWavesK = 8;
-  // K-steps per batch of loads: what the registers hold twice over with two workgroups on a CU where the
-  // grid has that many
-  constexpr int U = MT == 1 ? (FP4 ? 4 : 2) : (NT == 2 && MT == 2) ? 2 : 1;
-  constexpr int kStepBytes = FP4 ? 64 : 128;   // bytes of a row that one MFMA takes
-  static_assert(MT >= 1 && MT <= 4 && NT >= 1 && MT * NT <= kWavesK, "at most 64 rows of A; one wave per output tile at the end");
-  __shared__ v4f part[kWavesK][MT * NT][kWave];
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int l16 = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * (16 * NT);
-  const int k_steps = (K + 127) / 128;  // = chunks of four scale bytes per row of the blocked buffers
-  // Addresses are a base that is the same for the whole workgroup plus a 32-bit offset per lane (the
-  // host has checked that 255 rows of an operand span less than 4 GiB).  A workgroup's rows of B lie
-  // in one 128-row chunk of the blocked scales, and all of A's rows in the first.
-  auto scale_offset = [&](int row) { return (uint32_t)((row & 31) * 16 + ((row & 127) >> 5) * 4 + g); };
-  const uint8_t* const b0 = b + (int64_t)n0 * ldb;
-  const uint8_t* const sb0 = sfb + (int64_t)(n0 >> 7) * k_steps * 512;
-  uint32_t ob[NT], osb[NT], oa[MT], osa[MT];
-#pragma unroll
-  for (int j = 0; j < NT; ++j) {
-    const int brow = n0 + j * 16 + l16 < N ? n0 + j * 16 + l16 : N - 1;  // rows past the edge re-read the last one; never stored
-    ob[j] = (uint32_t)(brow - n0) * (uint32_t)ldb + g * 16;
-    osb[j] = scale_offset(brow);
-  }
-#pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int arow = t * 16 + l16 < M ? t * 16 + l16 : M - 1;
-    oa[t] = (uint32_t)arow * (uint32_t)lda + g * 16;
-    osa[t] = scale_offset(arow);
-  }
-  struct Batch {
-    v4i blo[NT][U], bhi[NT][U], alo[MT][U], ahi[MT][U];
-    int sb[NT][U], sa[MT][U];
-  };
-  const v4i zero4 = {0, 0, 0, 0};
-  auto load = [&](Batch& w, int first_step) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int k = first_step + u;
-      // What of the step lies inside K.  The scale byte of lane group g is that of the step's K-block g;
-      // its e2m1 elements are that block, but its e4m3 elements are the two 16-byte pieces at 16 g and
-      // 64 + 16 g, which belong to K-blocks g / 2 and 2 + g / 2.
-      const int left = K - k * 128;  // elements from this step on (none: the batch reaches past the last step)
-      const bool valid = g * 32 < left;
-      const bool valid_lo = FP4 ? valid : (g >> 1) * 32 < left, valid_hi = 64 + (g >> 1) * 32 < left;
-      const uint8_t* const bk = b0 + (int64_t)k * kStepBytes;
-      const uint8_t* const ak = a + (int64_t)k * kStepBytes;
-      const uint8_t* const sbk = sb0 + (int64_t)k * 512;
-      const uint8_t* const sak = sfa + (int64_t)k * 512;
-#pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        w.blo[j][u] = valid_lo ? *reinterpret_cast<const v4i*>(bk + ob[j]) : zero4;
-        if constexpr (!FP4) w.bhi[j][u] = valid_hi ? *reinterpret_cast<const v4i*>(bk + 64 + ob[j]) : zero4;
-        w.sb[j][u] = valid ? (int)sbk[osb[j]] : 0;
-      }
-#pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        w.alo[t][u] = valid_lo ? *reinterpret_cast<const v4i*>(ak + oa[t]) : zero4;
-        if constexpr (!FP4) w.ahi[t][u] = valid_hi ? *reinterpret_cast<const v4i*>(ak + 64 + oa[t]) : zero4;
-        w.sa[t][u] = valid ? (int)sak[osa[t]] : 0;
-      }
-    }
-  };
-  v4f acc[MT][NT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t)
-#pragma unroll
-    for (int j = 0; j < NT; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
-  auto compute = [&](const Batch& w) {
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        const v8i vb = FP4 ? __builtin_shufflevector(w.blo[j][u], zero4, 0, 1, 2, 3, 4, 5, 6, 7)
-                           : __builtin_shufflevector(w.blo[j][u], w.bhi[j][u], 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-          const v8i va = FP4 ? __builtin_shufflevector(w.alo[t][u], zero4, 0, 1, 2, 3, 4, 5, 6, 7)
-                             : __builtin_shufflevector(w.alo[t][u], w.ahi[t][u], 0, 1, 2, 3, 4, 5, 6, 7);
-          // B as the row operand: acc[t][j][v] = D[row 16 t + l16][column n0 + 16 j + 4 g + v]
-          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vb, va, acc[t][j], FP4 ? 4 : 0, FP4 ? 4 : 0, 0,
-                                                                       w.sb[j][u], 0, w.sa[t][u]);
-        }
-      }
-  };
-  // batches wave, wave + 8, ... of U steps each, over two register sets
-  const int batches = (k_steps + U - 1) / U;
-  int bi = wave;
-  if (bi < batches) {
-    Batch wa, wb;
-    load(wa, bi * U);
-    for (;;) {
-      bi += kWavesK;
-      if (bi >= batches) { compute(wa); break; }
-      load(wb, bi * U);
-      compute(wa);
-      bi += kWavesK;
-      if (bi >= batches) { compute(wb); break; }
-      load(wa, bi * U);
-      compute(wb);
-    }
-  }
-#pragma unroll
-  for (int t = 0; t < MT; ++t)
-#pragma unroll
-    for (int j = 0; j < NT; ++j) part[wave][t * NT + j][lane] = acc[t][j];
-  __syncthreads();
-  if (wave < MT * NT) {
-    v4f sum = part[0][wave][lane];
-#pragma unroll
-    for (int w = 1; w < kWavesK; ++w) sum += part[w][wave][lane];
-    const int m = (wave / NT) * 16 + l16, n = n0 + (wave % NT) * 16 + 4 * g;
-    if (m < M && n < N)  // N % 4 == 0: four columns or none
-      *reinterpret_cast<u32x2*>(out + (int64_t)m * ldo + n) = u32x2{pack_bf16x2(sum.x, sum.y), pack_bf16x2(sum.z, sum.w)};
-  }
-}
-
-// Where the kernel above beats the tiles (measured on MI355X, us, few rows against 128 x 128 tiles with
-// K shared through a workspace / without one; B rotated through 5 buffers so that it comes from HBM):
-// e2m1 16 x 8192 x 8192 11.7 against 21.7, 32 rows 14.7, 64 rows 18.9 against 22.1, 16 x 2048 x 8192 10.7
-// against 21.5, 16 x 16384 x 4096 11.4 against 13.0; e4m3 1 x 8192 x 8192 15.5 against 22.1 / 31.9,
-// 16 rows 21.4 against 20.0 / 31.8, 32 rows 24.2 against 23.1 / 32.3, 64 rows 31.9 against 23.8 / 35.0.
-// It loses where a workgroup reads more than twice as much of A as of B (64 x 4096 x 14336 e2m1: 25.6
-// against 19.0), where the columns make more than two workgroups per CU (16 x 28672 x 4096: 20.4
-// against 15.5 for e2m1, 34.3 against 30.5 for e4m3: a wave then lives for four K-steps and the launch is
-// all start-up), and for e4m3 against tiles that share K through a workspace.
-// 16-column tiles per wave: two (A's fragments used twice) once that still gives every CU a workgroup;
-// one for up to 8 rows of e4m3 (1 x 8192 x 8192: 15.5 against 19.7 us)
-template <bool FP4>
-int few_rows_tiles(int64_t M, int64_t N) {
-  const int forced = tuning("gemm.few_rows_tiles");
-  if (forced) return forced == 2 ? 2 : 1;
-  return N >= 32 * (int64_t)device_facts().cu_count && (FP4 || M > 8) ? 2 : 1;
-}
-
-template <bool FP4>
-bool few_rows_pays(int64_t M, int64_t N, int64_t K, bool have_workspace) {
-  const int64_t cus = device_facts().cu_count;
-  if (M > 64 || N < 8 * cus || K < 4096) return false;
-  const int tiles = few_rows_tiles<FP4>(M, N);
-  if (ceil_div(N, (int64_t)16 * tiles) > 2 * cus || M > 32 * tiles) return false;
-  return FP4 || !have_workspace || M <= 8;
-}
-
-template <bool FP4>
-int launch_skinny(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N,
-                  int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream) {
-  uint16_t* o = static_cast<uint16_t*>(out);
-  const bool two = few_rows_tiles<FP4>(M, N) == 2;
-  const unsigned grid = (unsigned)ceil_div(N, (int64_t)(two ? 32 : 16));
-#define DT_SKINNY(MT, NT) mx_skinny_kernel<FP4, MT, NT><<<grid, 512, 0, stream>>>(a, b, sfa, sfb, (int)M, (int)N, (int)K, lda, ldb, o, ldo)
-  if (M <= 16) { if (two) DT_SKINNY(1, 2); else DT_SKINNY(1, 1); }
-  else if (M <= 32) { if (two) DT_SKINNY(2, 2); else DT_SKINNY(2, 1); }
-  else if (M <= 48) { if (two) DT_SKINNY(3, 2); else DT_SKINNY(3, 1); }
-  else { if (two) DT_SKINNY(4, 2); else DT_SKINNY(4, 1); }
-#undef DT_SKINNY
-  return launch_status();
-}
-
 size_t split_workspace_bytes() { return kSplitTicketBytes + (size_t)device_facts().cu_count * kSplitTileBytes; }
 
 // Split-K factor for the 128 x 128 tiling.  A grid of a third of a workgroup per CU or less leaves
@@ -1035,8 +861,8 @@ int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb
   const uint8_t* B = static_cast<const uint8_t*>(b);
   hipStream_t s = as_hip(stream);
   const int variant = tuning("gemm.variant");
-  if ((variant == 9 && M <= 64) || (variant == 0 && few_rows_pays<FP4>(M, N, K, workspace != nullptr)))
-    return launch_skinny<FP4>(A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
+  if ((variant == 9 && M <= 64) || (variant == 0 && few_rows_pays(FP4, M, N, K, workspace != nullptr)))
+    return launch_few_rows(FP4, A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
   const int64_t tiles256 = ceil_div(M, 256) * ceil_div(N, 256);
   const bool big = variant == 2 || variant == 7 || (variant == 0 && tiles256 >= device_facts().cu_count / 2);
   // <tile M, tile N, waves M, waves N, LDS ring slots, e2m1 operands>

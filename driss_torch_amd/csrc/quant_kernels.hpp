@@ -130,11 +130,32 @@ __global__ __launch_bounds__(kBlock) void amax_kernel(const void* __restrict__ x
   m = block_umax<kBlock / kWave>(m, lds);
   stamp(2);
 
+  // Publishing the tensor's maximum: amax, the scales derived from it, into the workspace and to the caller
+  auto publish = [&](uint32_t bits) {
+    const float amax = as_f32(bits);
+    *reinterpret_cast<float*>(ws + kWsAmax) = amax;
+    if (amax_out) *amax_out = amax;
+    if constexpr (NSCALES > 0) {
+      float* wscale = reinterpret_cast<float*>(ws + kWsScale);
+      const float s0 = amax_to_scale(amax, fmax0);
+      wscale[0] = s0;
+      if (scale_out) scale_out[0] = s0;
+      if constexpr (NSCALES > 1) {
+        const float s1 = amax_to_scale(amax, fmax1);
+        wscale[1] = s1;
+        if (scale_out) scale_out[1] = s1;
+      }
+    }
+  };
   // One relaxed device-scope atomic max per workgroup carries the partial; a second one on the
   // ticket tells the last workgroup to arrive.  No fence is needed: the max is an atomic with
   // return, so it has been performed at the device's coherence point before the ticket is
   // taken, and ticket order is total.  (A release/acquire fence here costs a cache
   // write-back/invalidate per workgroup, which serialises: measured 10x the streaming time.)
+  // (Leaving each workgroup's maximum in a slot of its own with a store that writes through, and letting
+  // whoever then reads all slots marked publish the result, takes no read-modify-write at all, and is
+  // slower: the store's acknowledgement and the cache-missing loads take about 2 us each where an
+  // atomic with return takes 0.65 us.  8192 x 8192 bf16: 23.9 against 22.1 us; 1024 x 1024: 8.1 against 4.3.)
   uint32_t* ticket = reinterpret_cast<uint32_t*>(ws + kWsTicket);
   uint32_t* running = reinterpret_cast<uint32_t*>(ws + kWsRunning);
   if (tid == 0) {
@@ -147,20 +168,7 @@ __global__ __launch_bounds__(kBlock) void amax_kernel(const void* __restrict__ x
       // last to arrive: every other workgroup's max is already in `running`
       const uint32_t r = __hip_atomic_exchange(running, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // re-arm
       __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);                          // re-arm
-      const float amax = as_f32(r);
-      *reinterpret_cast<float*>(ws + kWsAmax) = amax;
-      if (amax_out) *amax_out = amax;
-      if constexpr (NSCALES > 0) {
-        float* wscale = reinterpret_cast<float*>(ws + kWsScale);
-        const float s0 = amax_to_scale(amax, fmax0);
-        wscale[0] = s0;
-        if (scale_out) scale_out[0] = s0;
-        if constexpr (NSCALES > 1) {
-          const float s1 = amax_to_scale(amax, fmax1);
-          wscale[1] = s1;
-          if (scale_out) scale_out[1] = s1;
-        }
-      }
+      publish(r);
     }
     stamp(3);
   }
@@ -363,21 +371,34 @@ __global__ __launch_bounds__(kBlock) void cast_kernel_unaligned(const void* __re
 template <int IN, int OUT, bool ROUND_BF16, bool ROUND_SCALE, bool PAIR>
 inline int launch_cast_impl(const void* x, int64_t numel, const float* scale, void* out, void* out2,
                             hipStream_t stream) {
-  // Batches of 4 loads per lane, software-pipelined (4..8 in flight), from ONE workgroup per CU: the best
-  // point of the measured grid {1, 2, 4 workgroups per CU} (8192^2 bf16 32.5 / 32.9 / 36.0 us, fp32 54.2 /
-  // 60.1 / 66 us, bf16 to both fp8 types 45.1 / 45.3 / 47.8 us); more in flight is slower
-  constexpr int kUnroll = 4;
+  // Large tensors: batches of 4 loads per lane, software-pipelined (4..8 in flight), from ONE workgroup per
+  // CU: the best point of the measured grid {1, 2, 4 workgroups per CU} (8192^2 bf16 32.5 / 32.9 / 36.0 us,
+  // fp32 54.2 / 60.1 / 66 us, bf16 to both fp8 types 45.1 / 45.3 / 47.8 us); more in flight is slower.
+  // Below 64 MiB of input, where the 3 us a launch costs whatever its size (launch, first round trip,
+  // drain) weigh more: batches of 2 from three workgroups per CU, which reach their full rate sooner
+  // (us, rotated buffers, batches of 4 and 1 workgroup per CU against this: bf16 4096^2 10.1 -> 9.6,
+  // 2048^2 4.2 -> 3.9; no difference from 64 MiB on).  The knobs force either (0 = by size).
   constexpr size_t kStoreAlign = IN == DT_F32 ? 4 : 8;
   uint8_t* o = static_cast<uint8_t*>(out);
   uint8_t* o2 = static_cast<uint8_t*>(out2);
   const bool fast = aligned(x, 16) && aligned(out, kStoreAlign) && (!PAIR || aligned(out2, kStoreAlign));
   if (fast) {
     const int64_t nvec = numel / InTraits<IN>::kVec, tail = numel % InTraits<IN>::kVec;
-    int grid = reduction_grid(nvec, kUnroll, PAIR ? "cast.pair_blocks_per_cu" : "cast.blocks_per_cu");
-    cast_kernel<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR, kUnroll><<<grid, kBlock, 0, stream>>>(x, nvec, tail, scale, o, o2);
+    const bool small = nvec * 16 < (int64_t)64 << 20;
+    const int unroll_knob = tuning("cast.unroll");
+    const int unroll = unroll_knob == 2 || unroll_knob == 4 ? unroll_knob : (small && !PAIR ? 2 : 4);
+    const char* const knob = PAIR ? "cast.pair_blocks_per_cu" : "cast.blocks_per_cu";
+    const int per_cu = tuning(knob) > 0 ? tuning(knob) : (small && !PAIR ? 3 : 1);
+    int64_t grid = ceil_div(nvec, (int64_t)kBlock * unroll);
+    if (grid > (int64_t)device_facts().cu_count * per_cu) grid = (int64_t)device_facts().cu_count * per_cu;
+    if (grid < 1) grid = 1;
+    if (unroll == 2) cast_kernel<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR, 2><<<(unsigned)grid, kBlock, 0, stream>>>(x, nvec, tail, scale, o, o2);
+    else cast_kernel<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR, 4><<<(unsigned)grid, kBlock, 0, stream>>>(x, nvec, tail, scale, o, o2);
   } else {
-    int grid = reduction_grid(numel / InTraits<IN>::kVec, 1, "cast.blocks_per_cu");
-    cast_kernel_unaligned<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR><<<grid, kBlock, 0, stream>>>(x, numel, scale, o, o2);
+    int64_t grid = ceil_div(numel / InTraits<IN>::kVec, (int64_t)kBlock);
+    if (grid > device_facts().cu_count) grid = device_facts().cu_count;
+    if (grid < 1) grid = 1;
+    cast_kernel_unaligned<IN, OUT, ROUND_BF16, ROUND_SCALE, PAIR><<<(unsigned)grid, kBlock, 0, stream>>>(x, numel, scale, o, o2);
   }
   return launch_status();
 }
