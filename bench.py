@@ -597,17 +597,58 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False, phases=None):
                  "bound": "mfma", "avg_us": round(us1, 2), "achieved_TFLOPs": round(flops / (us1 * 1e-6) / 1e12, 1),
                  "frac_of_fp8_peak": round(flops / (us1 * 1e-6) / 1e12 / FP8_PEAK_TFLOPS, 4), "flops": flops})
     del ones_a, ones_s
-    # two shapes off the 8192^3 grid, on row slices of the same operands (blocked scales are
-    # stored by 128-row chunks, so a row prefix of the operand owns a prefix of its scales)
-    for m_rows, n_rows, what in ((16, 8192, "16 rows: K shared between 4 workgroups per 128x128 tile"),
-                                 (1024, 8192, "128 tiles of 256x256 on 256 CUs: runs as 256 tiles of 256x128")):
-        sa_rows, sb_rows = -(-m_rows // 128) * 128 * (Kd // 32), -(-n_rows // 128) * 128 * (Kd // 32)
-        ops = (a_data[:m_rows], b_data[:n_rows], sfa[:sa_rows], sfb[:sb_rows], out[:m_rows, :n_rows])
-        gemm_small = bind(cabi, lambda: cabi.mx_fp8_bf16(*ops))
-        us = time_launches(lambda i: gemm_small(), 1, max(20, K // 2), 10)
-        fl = 2.0 * m_rows * n_rows * Kd
-        rows.append({"kernel": "mx_fp8_bf16", "workload": f"{m_rows}x{n_rows}x{Kd} e4m3 ({what})", "bound": "mfma",
-                     "avg_us": round(us, 2), "achieved_TFLOPs": round(fl / (us * 1e-6) / 1e12, 1), "flops": fl})
+    # shapes off the 8192^3 grid, on row slices of the same operands (blocked scales are stored by 128-row
+    # chunks, so a row prefix of the operand owns a prefix of its scales).  Each is warmed up for 40 ms first:
+    # under MFMA load the shader clock needs tens of milliseconds to settle, whatever the launch's length
+    def mfma_row(kernel, fn, ops, m_rows, n_rows, k_dim, what, peak, key):
+        g_ = bind(cabi, lambda: fn(*ops))
+        one = time_launches(lambda i: g_(), 1, 5, 2)
+        us_ = time_launches(lambda i: g_(), 1, max(50, K // 2), max(20, int(40e3 / max(one, 1.0))))
+        fl = 2.0 * m_rows * n_rows * k_dim
+        rows.append({"kernel": kernel, "workload": f"{m_rows}x{n_rows}x{k_dim} {what}", "bound": "mfma", "avg_us": round(us_, 2),
+                     "achieved_TFLOPs": round(fl / (us_ * 1e-6) / 1e12, 1), key: round(fl / (us_ * 1e-6) / 1e12 / peak, 4), "flops": fl})
+
+    for m_rows, n_rows, k_dim, what in ((1024, 8192, 8192, "e4m3 (128 tiles of 256x256 on 256 CUs: runs as 256 tiles of 256x128)"),
+                                        (4096, 4096, 4096, "e4m3 (256 tiles of 256x256: exactly one round of the chip)"),
+                                        (5120, 5120, 5120, "e4m3 (400 tiles: one round of 256x256 tiles, the other 144 as 256x128 halves or a second round)"),
+                                        (2048, 8192, 8192, "e4m3 (256 tiles, one round)")):
+        sa_rows = -(-m_rows // 128) * 128 * (Kd // 32)
+        sb_rows = -(-n_rows // 128) * 128 * (Kd // 32)
+        if k_dim == Kd:
+            ops = (a_data[:m_rows], b_data[:n_rows], sfa[:sa_rows], sfb[:sb_rows], out[:m_rows, :n_rows])
+        else:  # a shorter K: operands of their own (the blocked scale layout depends on K)
+            a_s, sa_s = cabi.mx_fp8_quantize(rnd((m_rows, k_dim), bf16, 11), 1, False, e4, cabi.SCALE_BLOCKED)
+            b_s, sb_s = cabi.mx_fp8_quantize(rnd((n_rows, k_dim), bf16, 12), 1, False, e4, cabi.SCALE_BLOCKED)
+            ops = (a_s, b_s, sa_s, sb_s, torch.empty((m_rows, n_rows), dtype=bf16, device=dev))
+        mfma_row("mx_fp8_bf16", cabi.mx_fp8_bf16, ops, m_rows, n_rows, k_dim, what, FP8_PEAK_TFLOPS, "frac_of_fp8_peak")
+
+    # Few rows (decode shapes): one pass over B, whose payload and scale bytes are the algorithmic bytes.  B rotates
+    # over enough operand sets to leave the 256 MB memory-side cache, so that every launch reads it from HBM;
+    # hot_cache_us is the same launch on one set.
+    def few_rows_row(kernel, fp4, m_rows):
+        nb = N * Kd // (2 if fp4 else 1) + N * Kd // 32
+        ns_ = nsets_for(nb)
+        sets_ = []
+        for i in range(ns_):
+            src = rnd((N, Kd), bf16, 20 + i)
+            sets_.append(cabi.mx_fp4_quantize(src, cabi.SCALE_BLOCKED) if fp4 else cabi.mx_fp8_quantize(src, 1, False, e4, cabi.SCALE_BLOCKED))
+            del src
+        a_src = rnd((m_rows, Kd), bf16, 1)
+        a_q, sa_q = cabi.mx_fp4_quantize(a_src, cabi.SCALE_BLOCKED) if fp4 else cabi.mx_fp8_quantize(a_src, 1, False, e4, cabi.SCALE_BLOCKED)
+        o_ = torch.empty((m_rows, N), dtype=bf16, device=dev)
+        fn = cabi.mx_fp4_bf16 if fp4 else cabi.mx_fp8_bf16
+        bound_ = [bind(cabi, lambda bq=bq, sq=sq: fn(a_q, bq, sa_q, sq, o_)) for bq, sq in sets_]
+        us_ = time_launches(lambda i: bound_[i](), ns_, max(50, K // 2), 20)
+        hot_ = time_launches(lambda i: bound_[0](), 1, max(50, K // 2), 20)
+        rows.append({"kernel": kernel, "workload": f"{m_rows}x{N}x{Kd} {'e2m1' if fp4 else 'e4m3'} (few rows: B straight from memory into the "
+                     "MFMA's registers, A through LDS, K shared between a workgroup's eight waves)", "bound": "hbm", "avg_us": round(us_, 2),
+                     "achieved_GBs": round(nb / us_ / 1e3, 1), "frac_of_8TBs": round(nb / us_ / 1e3 / HBM_PEAK_GBS, 4),
+                     "hot_cache_us": round(hot_, 2), "algorithmic_bytes": nb, "buffer_sets": ns_})
+        del sets_, bound_
+        torch.cuda.empty_cache()
+
+    few_rows_row("mx_fp8_bf16", False, 16)
+    few_rows_row("mx_fp8_bf16", False, 64)
     # MXFP4 GEMM, same shape: the MXFP4 cast of the same N(0,1) operands, scales blocked by the cast
     del a_data, b_data
     a4, s4a = cabi.mx_fp4_quantize(rnd((M, Kd), bf16, 1), cabi.SCALE_BLOCKED)
@@ -618,15 +659,9 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False, phases=None):
     rows.append({"kernel": "mx_fp4_bf16", "workload": "8192^3 e2m1 x e2m1, E8M0 block-32 scales -> bf16",
                  "bound": "mfma", "avg_us": round(us, 2), "achieved_TFLOPs": round(tf, 1),
                  "frac_of_fp4_peak": round(tf / FP4_PEAK_TFLOPS, 4), "flops": flops})
-    # 16 rows of the same operands: one pass over B (its payload and scale bytes are the algorithmic
-    # bytes; one operand set, 33 MB, so the memory-side cache may hold it); the library's kernel for few rows
-    ops4 = (a4[:16], b4, s4a[:128 * (Kd // 32)], s4b, out[:16])
-    gemm4s = bind(cabi, lambda: cabi.mx_fp4_bf16(*ops4))
-    us = time_launches(lambda i: gemm4s(), 1, max(20, K // 2), 10)
-    nbytes = N * Kd // 2 + N * Kd // 32
-    rows.append({"kernel": "mx_fp4_bf16", "workload": f"16x{N}x{Kd} e2m1 (few rows: 32 columns per workgroup, K shared between its "
-                 "eight waves, operands straight from memory into registers)", "bound": "hbm", "avg_us": round(us, 2),
-                 "achieved_GBs": round(nbytes / us / 1e3, 1), "algorithmic_bytes": nbytes, "buffer_sets": 1})
+    del a4, b4, s4a, s4b
+    torch.cuda.empty_cache()
+    few_rows_row("mx_fp4_bf16", True, 16)
     return rows
 
 

@@ -30,7 +30,7 @@ HIP_LIB = LIB / "libdriss_torch_hip.so"
 TORCH_LIB = LIB / "libdriss_torch.so"
 PHASES_HIP_LIB = LIB / "libdriss_torch_hip_phases.so"  # made on request only (--phase-log)
 
-HIP_SOURCES = ["mx_fp8_bf16.hip", "mx_few_rows.hip", "abi_common.hip", "amax.hip", "saturated_cast.hip",
+HIP_SOURCES = ["mx_fp8_bf16.hip", "mx_fp4_bf16.hip", "mx_few_rows.hip", "abi_common.hip", "amax.hip", "saturated_cast.hip",
                "dynamic_scaled_quant.hip", "mx_cast.hip"]
 
 HIPCC_FLAGS = [

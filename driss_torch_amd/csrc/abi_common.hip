@@ -46,7 +46,6 @@ struct Knob {
 Knob g_knobs[] = {
     {"gemm.few_rows_tiles", 0},
     {"gemm.few_rows_stagger", 1},
-    {"gemm.few_rows_waves", 0},
     {"gemm.few_rows_steps", 0},
     {"gemm.few_rows_per_cu", 0},
     {"amax.blocks_per_cu", 1},

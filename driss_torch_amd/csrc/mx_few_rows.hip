@@ -1,21 +1,35 @@
 // The block-scaled GEMM for few rows (M <= 64): out[M,N] = (A 2^sfa)(B 2^sfb)^T with e4m3 or e2m1 operands.
 //
 // Such a problem is one pass over B, and a tile with a 128- or 256-row A panel would idle most of its
-// MFMAs and leave the chip to a handful of workgroups.  Here a workgroup of WAVES waves owns a group of
+// MFMAs and leave the chip to a handful of workgroups.  Here a workgroup of 8 waves owns a group of
 // 16 NT rows of B (= output columns) at a time and every row of A; its waves share K between them in
-// turns of U K-steps of 128 elements, so the workgroup as a whole walks 16 NT whole rows of B.  Nothing
-// goes through LDS on the way in: a lane's part of an MFMA operand is two 16-byte pieces of one row, 64
-// bytes apart (one piece with e2m1), and the four lanes that share a row read 64 contiguous bytes of it
-// per load instruction (bytes 16 g .. of the step in lane group g); the E8M0 byte of a lane is one byte of
-// the blocked scale buffer.  A's rows come out of the L2 the same way (every workgroup reads all of A: M x K
-// bytes, a few hundred KiB).  A batch of U steps is in registers while the next one's loads are in flight.
-// The waves' partial sums meet in LDS and are added in wave order; one wave per 16 x 16 output tile writes
-// it.  K-blocks past the end of K (K % 128 != 0) enter as zeros with a scale of 2^-127.
+// turns of UP panel steps of 128 bytes, so the workgroup as a whole walks 16 NT whole rows of B.
+//
+// B goes straight from memory into the registers the MFMA takes: a lane's part of an operand is two
+// 16-byte pieces of one row, 64 bytes apart, and the four lanes that share a row read 64 contiguous bytes
+// of it per load instruction; the E8M0 byte of a lane is one byte of the blocked scale buffer.
+//
+// A comes out of the L2 (every workgroup reads all of A: M x K bytes, a few hundred KiB), and how it is
+// asked for matters more than B's stream: loaded the way B is, every load instruction asks the L2 for 16
+// half lines, and a launch of 64 rows spends half its time on them (measured by leaving A's loads out).
+// So a wave moves the rows of A it is about to use into a region of LDS of its own with
+// global_load_lds_dwordx4 -- 8 rows x 128 bytes, whole lines, per instruction, no registers -- and reads
+// its fragments from there (16-byte chunks XOR-swizzled inside each group of 8 rows: conflict-free),
+// and A's blocked scale chunks travel the same way.  No other wave reads that region: no barrier.
+//
+// A batch (UP steps) is in registers / LDS while the next one's loads are in flight.  All of a batch's
+// memory instructions are written as assembly and counted by hand (one s_waitcnt per batch): the
+// compiler does not see the LDS-DMA loads, and its own counts would make a batch wait for part of the
+// next one.  The waves' partial sums meet in LDS and are added in wave order; one wave per 16 x 16
+// output tile writes it.  K-blocks past the end of K (K % 128 != 0) enter with a scale of 2^-127 on both
+// sides, which leaves the sums as they are; their payload bytes are valid bytes of the same row read again.
 //
 // The grid is persistent: a workgroup takes the column groups b, b + grid, ... and the batch it loads
 // ahead may belong to its next group, so those loads are in flight under the reduction and the stores of
 // the group in hand.
 #include "mx_few_rows.hpp"
+
+#include <atomic>
 
 #include "dt_device.hpp"
 #include "dt_host.hpp"
@@ -28,28 +42,81 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-template <bool FP4, int MT, int NT, int WAVES, int U>
-__global__ __launch_bounds__(WAVES* kWave) void mx_few_rows_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
-                                                                  const uint8_t* __restrict__ sfa, const uint8_t* __restrict__ sfb,
-                                                                  int M, int N, int K, int64_t lda, int64_t ldb,
-                                                                  uint16_t* __restrict__ out, int64_t ldo, int groups, int stagger) {
-  constexpr int kStepBytes = FP4 ? 64 : 128;  // bytes of a row that one MFMA takes
-  static_assert(MT >= 1 && MT <= 4 && NT >= 1 && NT <= 2, "at most 64 rows of A, 32 columns per group");
-  __shared__ v4f part[WAVES][MT * NT][kWave];
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+constexpr int kFewWaves = 8;
+
+// 16 bytes / one byte per lane at a base that is the same for the whole wave plus a 32-bit lane offset.
+// The value arrives later: nothing may look at it before wait_loads.
+__device__ __forceinline__ v4i load16_async(uint32_t lane_off, const uint8_t* wave_base) {
+  v4i r;
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(lane_off), "s"(wave_base) : "memory");
+  return r;
+}
+__device__ __forceinline__ int load_byte_async(uint32_t lane_off, const uint8_t* wave_base) {
+  int r;
+  asm volatile("global_load_ubyte %0, %1, %2" : "=v"(r) : "v"(lane_off), "s"(wave_base) : "memory");
+  return r;
+}
+// 16 bytes per lane from memory into LDS at lds_addr + 16 * lane, without a register in between
+__device__ __forceinline__ void load16_to_lds_async(uint32_t lds_addr, uint32_t lane_off, const uint8_t* wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(lane_off), "s"(wave_base) : "memory");
+}
+// until at most N of this wave's loads are outstanding (they complete in the order they were issued)
+template <int N>
+__device__ __forceinline__ void wait_loads() {
+  static_assert(N >= 0 && N < 64, "the counter has 6 bits");
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+template <bool FP4, int MT, int NT, int UP>
+__global__ __launch_bounds__(kFewWaves* kWave) void mx_few_rows_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
+                                                                     const uint8_t* __restrict__ sfa, const uint8_t* __restrict__ sfb,
+                                                                     int M, int N, int K, int64_t lda, int64_t ldb,
+                                                                     uint16_t* __restrict__ out, int64_t ldo, int groups, int stagger) {
+  constexpr int WAVES = kFewWaves;
+  constexpr int KC = FP4 ? 2 : 1;  // MFMAs, and blocked scale chunks, per panel step of 128 bytes of a row
+  static_assert(MT >= 1 && MT <= 4 && NT >= 1 && NT <= 2 && UP >= 1, "at most 64 rows of A, 32 columns per group");
+  // LDS of a wave: two sets of [A rows of a batch: step, tile, half of 8 rows, 8 rows x 128 B][A scale chunks of the batch]
+  constexpr int kPanel = UP * MT * 2048;
+  constexpr int kScaleLoads = (UP * KC + 1) / 2;  // of 1 KiB = two scale chunks
+  constexpr int kSetBytes = kPanel + kScaleLoads * 1024, kWaveBytes = 2 * kSetBytes;
+  static_assert(MT * NT * 1024 <= kPanel, "a wave parks its sums in the set it has just used up");
+  // loads of a batch, in the order they are issued
+  constexpr int kLoadsPerBatch = UP * NT * 2 + UP * NT * KC + UP * MT * 2 + kScaleLoads;
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x / kWave);
   const int l16 = lane & 15, g = lane >> 4;
-  const int k_steps = (K + 127) / 128;  // = chunks of four scale bytes per row of the blocked buffers
-  // Addresses are a base that is the same for the whole workgroup plus a 32-bit offset per lane (the
-  // host has checked that 255 rows of an operand span less than 4 GiB).  A group's rows of B lie in one
-  // 128-row chunk of the blocked scales, and all of A's rows in the first.
-  auto scale_offset = [&](int row) { return (uint32_t)((row & 31) * 16 + ((row & 127) >> 5) * 4 + g); };
-  uint32_t oa[MT], osa[MT];
+  const uint32_t lds_wave = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds + (uint32_t)wave * kWaveBytes;
+  uint8_t* const my_lds = lds + wave * kWaveBytes;
+  const int k_bytes = FP4 ? K / 2 : K;                 // of a row
+  const int p_steps = (k_bytes + 127) / 128;           // panel steps
+  const int k_chunks = (K + 127) / 128;                // blocked scale chunks per 128 rows
+  const int tail_p = (k_bytes % 128) ? p_steps - 1 : -1;  // a partly filled last step
+  const int tail_chunks = (k_bytes % 128) / 16;
+
+  // ---- per-lane offsets.  A, as LDS-DMA: lane L fills row L / 8, chunk position L % 8 of a group of 8
+  // rows, i.e. it fetches logical chunk (L % 8) ^ (L / 8) of that row; in a partly filled step a chunk
+  // past the end reads chunk c % (valid chunks) again (never the next row, never past the tensor).
+  const int drow = lane >> 3, dchunk = (lane & 7) ^ drow;
+  const uint32_t a_tail_adj = tail_chunks > 0 ? (uint32_t)(dchunk - dchunk % tail_chunks) * 16u : 0u;
+  uint32_t oa[MT][2];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int arow = t * 16 + l16 < M ? t * 16 + l16 : M - 1;
-    oa[t] = (uint32_t)arow * (uint32_t)lda + g * 16;
-    osa[t] = scale_offset(arow);
-  }
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int r = t * 16 + h * 8 + drow;
+      oa[t][h] = (uint32_t)(r < M ? r : M - 1) * (uint32_t)lda + dchunk * 16;
+    }
+  // A's fragments in LDS: row l16 of a tile = group l16 / 8, row l16 % 8; logical chunks g and 4 + g
+  const uint32_t frag_lo = (l16 >> 3) * 1024 + (l16 & 7) * 128 + ((g ^ (l16 & 7)) << 4), frag_hi = frag_lo ^ 64u;
+  // a row's scale word inside a 512-byte chunk of 128 rows; the lane's own byte is K-block g
+  auto scale_offset = [&](int row) { return (uint32_t)((row & 31) * 16 + ((row & 127) >> 5) * 4 + g); };
+  uint32_t osa[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) osa[t] = scale_offset(t * 16 + l16 < M ? t * 16 + l16 : M - 1);
+  // B: the two pieces of a lane (bytes 16 g and 64 + 16 g of the step); in a partly filled step a piece
+  // past the end reads the row's first piece of the step again
+  const bool lo_in_tail = g < tail_chunks, hi_in_tail = 4 + g < tail_chunks;
   // what of B depends on the column group
   struct Group {
     const uint8_t *b0, *sb0;
@@ -59,51 +126,53 @@ __global__ __launch_bounds__(WAVES* kWave) void mx_few_rows_kernel(const uint8_t
     Group q;
     const int n0 = grp * (16 * NT);
     q.b0 = b + (int64_t)n0 * ldb;
-    q.sb0 = sfb + (int64_t)(n0 >> 7) * k_steps * 512;
+    q.sb0 = sfb + (int64_t)(n0 >> 7) * k_chunks * 512;
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       const int brow = n0 + j * 16 + l16 < N ? n0 + j * 16 + l16 : N - 1;  // rows past the edge re-read the last one; never stored
-      q.ob[j] = (uint32_t)(brow - n0) * (uint32_t)ldb + g * 16;
+      q.ob[j] = (uint32_t)(brow - n0) * (uint32_t)ldb;
       q.osb[j] = scale_offset(brow);
     }
     return q;
   };
   struct Batch {
-    v4i blo[NT][U], bhi[NT][U], alo[MT][U], ahi[MT][U];
-    int sb[NT][U], sa[MT][U];
+    v4i blo[NT][UP], bhi[NT][UP];
+    int sb[NT][UP][KC];
   };
-  const v4i zero4 = {0, 0, 0, 0};
-#ifdef DT_FEW_ROWS_STREAM_B
-  auto ld_b = [](const v4i* p) { return __builtin_nontemporal_load(p); };
-#else
-  auto ld_b = [](const v4i* p) { return *p; };
-#endif
-  auto load = [&](Batch& w, const Group& q, int first_step) {
+  // Everything a batch needs is sent for here: kLoadsPerBatch instructions whatever the batch (a step
+  // past the last one reads the last one again and counts as nothing, see consume)
+  auto issue = [&](Batch& w, int set, const Group& q, int first_step) {
+    const uint32_t lds_set = lds_wave + (uint32_t)set * kSetBytes;
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int k = first_step + u;
-      // What of the step lies inside K.  The scale byte of lane group g is that of the step's K-block g;
-      // its e2m1 elements are that block, but its e4m3 elements are the two 16-byte pieces at 16 g and
-      // 64 + 16 g, which belong to K-blocks g / 2 and 2 + g / 2.
-      const int left = K - k * 128;  // elements from this step on (none: the batch reaches past the last step)
-      const bool valid = g * 32 < left;
-      const bool valid_lo = FP4 ? valid : (g >> 1) * 32 < left, valid_hi = 64 + (g >> 1) * 32 < left;
-      const uint8_t* const bk = q.b0 + (int64_t)k * kStepBytes;
-      const uint8_t* const ak = a + (int64_t)k * kStepBytes;
-      const uint8_t* const sbk = q.sb0 + (int64_t)k * 512;
-      const uint8_t* const sak = sfa + (int64_t)k * 512;
+    for (int u = 0; u < UP; ++u) {
+      const int p = first_step + u < p_steps ? first_step + u : p_steps - 1;
+      const bool tail = p == tail_p;
+      const uint8_t* const bk = q.b0 + (int64_t)p * 128;
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
-        w.blo[j][u] = valid_lo ? ld_b(reinterpret_cast<const v4i*>(bk + q.ob[j])) : zero4;
-        if constexpr (!FP4) w.bhi[j][u] = valid_hi ? ld_b(reinterpret_cast<const v4i*>(bk + 64 + q.ob[j])) : zero4;
-        w.sb[j][u] = valid ? (int)sbk[q.osb[j]] : 0;
+        w.blo[j][u] = load16_async(q.ob[j] + ((tail && !lo_in_tail) ? 0u : (uint32_t)g * 16u), bk);
+        w.bhi[j][u] = load16_async(q.ob[j] + ((tail && !hi_in_tail) ? 0u : 64u + (uint32_t)g * 16u), bk);
       }
 #pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        w.alo[t][u] = valid_lo ? *reinterpret_cast<const v4i*>(ak + oa[t]) : zero4;
-        if constexpr (!FP4) w.ahi[t][u] = valid_hi ? *reinterpret_cast<const v4i*>(ak + 64 + oa[t]) : zero4;
-        w.sa[t][u] = valid ? (int)sak[osa[t]] : 0;
+      for (int c = 0; c < KC; ++c) {
+        const int kc = p * KC + c < k_chunks ? p * KC + c : k_chunks - 1;
+        const uint8_t* const sbk = q.sb0 + (int64_t)kc * 512;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) w.sb[j][u][c] = load_byte_async(q.osb[j], sbk);
       }
+      const uint8_t* const ak = a + (int64_t)p * 128;
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          load16_to_lds_async(lds_set + ((u * MT + t) * 2 + h) * 1024, oa[t][h] - (tail ? a_tail_adj : 0u), ak);
+    }
+    // A's scale chunks of the batch are neighbours in the blocked buffer: 1 KiB = two chunks per instruction
+    const int c0 = first_step * KC;
+#pragma unroll
+    for (int i = 0; i < kScaleLoads; ++i) {
+      const int kc = c0 + 2 * i + (lane >> 5);
+      load16_to_lds_async(lds_set + kPanel + i * 1024, (uint32_t)(kc < k_chunks ? kc : k_chunks - 1) * 512u + (lane & 31) * 16u, sfa);
     }
   };
   v4f acc[MT][NT];
@@ -113,130 +182,191 @@ __global__ __launch_bounds__(WAVES* kWave) void mx_few_rows_kernel(const uint8_t
 #pragma unroll
       for (int j = 0; j < NT; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
   };
-  auto compute = [&](const Batch& w) {
+  // The batch has arrived (the caller has waited): MFMAs with A's fragments and scale bytes out of LDS
+  auto consume = [&](Batch& w, int set, int first_step) {
+    const uint8_t* const set_lds = my_lds + set * kSetBytes;
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < UP; ++u) {
 #pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        const v8i vb = FP4 ? __builtin_shufflevector(w.blo[j][u], zero4, 0, 1, 2, 3, 4, 5, 6, 7)
-                           : __builtin_shufflevector(w.blo[j][u], w.bhi[j][u], 0, 1, 2, 3, 4, 5, 6, 7);
+      for (int j = 0; j < NT; ++j) {  // from here on the loaded values may be looked at
+        asm volatile("" : "+v"(w.blo[j][u]), "+v"(w.bhi[j][u]));
 #pragma unroll
-        for (int t = 0; t < MT; ++t) {
-          const v8i va = FP4 ? __builtin_shufflevector(w.alo[t][u], zero4, 0, 1, 2, 3, 4, 5, 6, 7)
-                             : __builtin_shufflevector(w.alo[t][u], w.ahi[t][u], 0, 1, 2, 3, 4, 5, 6, 7);
-          // B as the row operand: acc[t][j][v] = D[row 16 t + l16][column n0 + 16 j + 4 g + v]
-          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vb, va, acc[t][j], FP4 ? 4 : 0, FP4 ? 4 : 0, 0,
-                                                                       w.sb[j][u], 0, w.sa[t][u]);
+        for (int c = 0; c < KC; ++c) asm volatile("" : "+v"(w.sb[j][u][c]));
+      }
+      // elements of K from this step on; the lane's K-block of MFMA c starts 128 c + 32 g elements in
+      const int left = K - (first_step + u) * (FP4 ? 256 : 128);
+#pragma unroll
+      for (int c = 0; c < KC; ++c) {
+        const bool valid = c * 128 + g * 32 < left;
+        int sa[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) sa[t] = valid ? (int)set_lds[kPanel + (u * KC + c) * 512 + osa[t]] : 0;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          const int sb = valid ? w.sb[j][u][c] : 0;
+          const v8i vb = FP4 ? __builtin_shufflevector(c == 0 ? w.blo[j][u] : w.bhi[j][u], v4i{0, 0, 0, 0}, 0, 1, 2, 3, 4, 5, 6, 7)
+                             : __builtin_shufflevector(w.blo[j][u], w.bhi[j][u], 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+          for (int t = 0; t < MT; ++t) {
+            const uint8_t* const f = set_lds + (u * MT + t) * 2048;
+            const v4i alo = *reinterpret_cast<const v4i*>(f + frag_lo), ahi = *reinterpret_cast<const v4i*>(f + frag_hi);
+            const v8i va = FP4 ? __builtin_shufflevector(c == 0 ? alo : ahi, v4i{0, 0, 0, 0}, 0, 1, 2, 3, 4, 5, 6, 7)
+                               : __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7);
+            // B as the row operand: acc[t][j][v] = D[row 16 t + l16][column n0 + 16 j + 4 g + v]
+            acc[t][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vb, va, acc[t][j], FP4 ? 4 : 0, FP4 ? 4 : 0, 0, sb, 0, sa[t]);
+          }
         }
       }
+    }
   };
-  // The end of a group: the waves' sums meet in LDS and are added in wave order (the same sum whatever
-  // the timing); wave t takes the output tiles t, t + WAVES, ...
-  auto finish = [&](int grp) {
+  // The end of a group: every wave parks its sums in the set it has just used up (the other one may be
+  // receiving the next batch), they are added in wave order (the same sum whatever the timing), and
+  // wave t writes the output tiles t, t + 8, ...
+  auto finish = [&](int grp, int set) {
+    v4f* const mine = reinterpret_cast<v4f*>(my_lds + set * kSetBytes);
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
-      for (int j = 0; j < NT; ++j) part[wave][t * NT + j][lane] = acc[t][j];
+      for (int j = 0; j < NT; ++j) mine[(t * NT + j) * kWave + lane] = acc[t][j];
     __syncthreads();
     const int n0 = grp * (16 * NT);
 #pragma unroll
     for (int tile0 = 0; tile0 < MT * NT; tile0 += WAVES) {
       const int tile = tile0 + wave;
       if (tile < MT * NT) {
-        v4f sum = part[0][tile][lane];
+        v4f sum = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int w = 1; w < WAVES; ++w) sum += part[w][tile][lane];
+        for (int w = 0; w < WAVES; ++w) sum += reinterpret_cast<const v4f*>(lds + w * kWaveBytes + set * kSetBytes)[tile * kWave + lane];
         const int m = (tile / NT) * 16 + l16, n = n0 + (tile % NT) * 16 + 4 * g;
         if (m < M && n < N)  // N % 4 == 0: four columns or none
           *reinterpret_cast<u32x2*>(out + (int64_t)m * ldo + n) = u32x2{pack_bf16x2(sum.x, sum.y), pack_bf16x2(sum.z, sum.w)};
       }
     }
-    __syncthreads();  // before anybody parks the next group's sums
+    __syncthreads();  // before anybody's next batch lands in that set
   };
 
-  // This wave's batches of a group: wave, wave + WAVES, ... of U steps each.  The workgroups do not all
-  // start at the front of their rows: group number grp begins `rot` batches in and wraps around, so that
-  // at any moment the chip's loads are spread over the whole length of the rows (the rows are a power of
-  // two apart in most problems: with every workgroup at the same K offset the requests of the moment
-  // fall on a fraction of the memory channels).
-  const int batches = (k_steps + U - 1) / U;
+  // A wave's batches of a group: wave, wave + 8, ... of UP steps each, the same number for every wave
+  // (one past the last batch is sent for like any other and counts as nothing).  The workgroups do
+  // not all start at the front of their rows: group number grp begins `rot` batches in and wraps around,
+  // so that at any moment the chip's loads are spread over the whole length of the rows.
+  const int batches = (p_steps + UP - 1) / UP, per_wave = (batches + WAVES - 1) / WAVES;
   auto first_step_of = [&](int grp, int i) {
-    const int r = i + (stagger ? (int)(((unsigned)grp * 5u) % (unsigned)batches) : 0);
-    return (r >= batches ? r - batches : r) * U;
+    const int bi = wave + i * WAVES;
+    if (bi >= batches) return p_steps;
+    const int r = bi + (stagger ? (int)(((unsigned)grp * 5u) % (unsigned)batches) : 0);
+    return (r >= batches ? r - batches : r) * UP;
   };
-  // The sequence of (group, batch) pairs of this wave, over two register sets: the pair after the one
-  // being computed is already on its way, also across the end of a group.
-  int grp = blockIdx.x, bi = wave;
-  auto advance = [&](int& gq, int& bq) {  // the pair after (gq, bq); gq >= groups: none
-    bq += WAVES;
-    if (bq >= batches) { bq = wave; gq += gridDim.x; }
-  };
-  if (wave >= batches) {  // fewer batches than waves: this wave only takes part in the reductions
-    for (; grp < groups; grp += gridDim.x) { clear(); finish(grp); }
-    return;
-  }
+  // The sequence of (group, batch) pairs of this wave over two sets of registers and LDS: the pair after
+  // the one being computed is already on its way, also across the end of a group.
+  int grp = blockIdx.x, i = 0;
   if (grp >= groups) return;  // (the whole workgroup)
+  auto advance = [&](int& gq, int& iq) {  // the pair after (gq, iq); gq >= groups: none
+    if (++iq == per_wave) { iq = 0; gq += gridDim.x; }
+  };
   Batch wa, wb;
   Group q = group_at(grp);
-  load(wa, q, first_step_of(grp, bi));
+  int step = first_step_of(grp, i);
+  issue(wa, 0, q, step);
   clear();
   for (;;) {
-    // ---- wa holds (grp, bi): send for its successor into wb, compute wa
-    int g2 = grp, b2 = bi;
-    advance(g2, b2);
+    // ---- set 0 holds (grp, i): send for its successor into set 1, then compute set 0
+    int g2 = grp, i2 = i;
+    advance(g2, i2);
     Group q2 = q;
-    if (g2 != grp && g2 < groups) q2 = group_at(g2);
-    if (g2 < groups) load(wb, q2, first_step_of(g2, b2));
-    compute(wa);
-    if (g2 != grp) { finish(grp); clear(); }
+    int step2 = 0;
+    if (g2 < groups) {
+      if (g2 != grp) q2 = group_at(g2);
+      step2 = first_step_of(g2, i2);
+      issue(wb, 1, q2, step2);
+      wait_loads<kLoadsPerBatch>();
+    } else {
+      wait_loads<0>();
+    }
+    consume(wa, 0, step);
+    if (g2 != grp) { finish(grp, 0); clear(); }
     if (g2 >= groups) break;
-    grp = g2; bi = b2; q = q2;
-    // ---- wb holds (grp, bi): the same with the roles of the sets swapped
-    advance(g2, b2);
-    if (g2 != grp && g2 < groups) q2 = group_at(g2);
-    if (g2 < groups) load(wa, q2, first_step_of(g2, b2));
-    compute(wb);
-    if (g2 != grp) { finish(grp); clear(); }
+    grp = g2; i = i2; q = q2; step = step2;
+    // ---- set 1 holds (grp, i): the same with the roles of the sets swapped
+    advance(g2, i2);
+    if (g2 < groups) {
+      if (g2 != grp) q2 = group_at(g2);
+      step2 = first_step_of(g2, i2);
+      issue(wa, 0, q2, step2);
+      wait_loads<kLoadsPerBatch>();
+    } else {
+      wait_loads<0>();
+    }
+    consume(wb, 1, step);
+    if (g2 != grp) { finish(grp, 1); clear(); }
     if (g2 >= groups) break;
-    grp = g2; bi = b2; q = q2;
+    grp = g2; i = i2; q = q2; step = step2;
   }
 }
 
-// Shape of the launch for a problem: 16-column tiles per group (NT), waves per workgroup, K-steps per batch
+// Shape of the launch for a problem: 16-column tiles per group (NT), panel steps per batch (UP)
 struct Plan {
-  int nt, waves, steps;
+  int nt, up;
 };
+
+constexpr size_t few_rows_lds_bytes(bool fp4, int mt, int up) {
+  return (size_t)kFewWaves * 2 * ((size_t)up * mt * 2048 + (size_t)((up * (fp4 ? 2 : 1) + 1) / 2) * 1024);
+}
+constexpr size_t kLdsLimit = 160 * 1024;
 
 Plan plan_for(bool fp4, int64_t M, int64_t N) {
   Plan p;
   const int tiles = tuning("gemm.few_rows_tiles");
   p.nt = tiles ? (tiles == 2 ? 2 : 1) : (N >= 32 * (int64_t)device_facts().cu_count && (fp4 || M > 8) ? 2 : 1);
   const int mt = (int)((M + 15) / 16);
-  const int waves = tuning("gemm.few_rows_waves");
-  p.waves = waves == 4 ? 4 : 8;
-  int steps = tuning("gemm.few_rows_steps");
-  if (steps != 1 && steps != 2 && steps != 4) steps = mt == 1 ? (fp4 ? 4 : 2) : (p.nt == 2 && mt == 2) ? 2 : 1;
-  // two register sets of (NT + MT) U fragments of 4 (e2m1) or 8 registers must leave room for the rest
-  while (steps > 1 && 2 * (p.nt + mt) * steps * (fp4 ? 4 : 8) > 144) steps /= 2;
-  p.steps = steps;
+  int up = tuning("gemm.few_rows_steps");
+  if (up != 1 && up != 2) up = mt == 1 ? 2 : 1;
+  if (up == 2 && (mt > 2 || few_rows_lds_bytes(fp4, mt, 2) >= kLdsLimit)) up = 1;
+  p.up = up;
   return p;
+}
+
+template <bool FP4, int MT, int NT, int UP>
+int launch_instance(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N, int64_t K,
+                    int64_t lda, int64_t ldb, uint16_t* out, int64_t ldo, int64_t groups, int64_t grid, int stagger,
+                    hipStream_t stream) {
+  constexpr size_t kLds = few_rows_lds_bytes(FP4, MT, UP);
+  static_assert(kLds <= kLdsLimit, "two sets per wave fit the CU's LDS");
+  auto kernel = mx_few_rows_kernel<FP4, MT, NT, UP>;
+  if (kLds > 64 * 1024) {  // once per instantiation and device
+    static std::atomic<bool> allowed[16];
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    const bool tracked = dev >= 0 && dev < 16;
+    if (!tracked || !allowed[dev].load(std::memory_order_relaxed)) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds) != hipSuccess)
+        return DT_ERR_LAUNCH;
+      if (tracked) allowed[dev].store(true, std::memory_order_relaxed);
+    }
+  }
+  kernel<<<(unsigned)grid, kFewWaves * kWave, kLds, stream>>>(a, b, sfa, sfb, (int)M, (int)N, (int)K, lda, ldb, out, ldo, (int)groups,
+                                                            stagger);
+  return launch_status();
 }
 
 }  // namespace
 
-// Where the kernel above beats the tiles (measured on MI355X, us, few rows against 128 x 128 tiles with
-// K shared through a workspace / without one; B rotated through 5 buffers so that it comes from HBM):
-// e2m1 16 x 8192 x 8192 11.7 against 21.7, 32 rows 14.7, 64 rows 18.9 against 22.1, 16 x 2048 x 8192 10.7
-// against 21.5, 16 x 16384 x 4096 11.4 against 13.0; e4m3 1 x 8192 x 8192 15.5 against 22.1 / 31.9,
-// 16 rows 21.4 against 20.0 / 31.8, 32 rows 24.2 against 23.1 / 32.3, 64 rows 31.9 against 23.8 / 35.0.
-// It loses where a workgroup reads more than twice as much of A as of B (64 x 4096 x 14336 e2m1: 25.6
-// against 19.0), and for e4m3 against tiles that share K through a workspace.
+// Where the kernel above beats the 128 x 128 tiles that share K through a workspace (measured on MI355X,
+// us, B rotated through enough buffers that it comes from HBM; few rows / tiles):
+//   8192 x 8192:  e4m3 M = 8 16.9 / 19.6, 16 16.4 / 19.5, 32 18.8 / 20.0, 64 22.3 / 21.6; e2m1 10.7 / 23.7, 10.9 / 23.7, 12.2 / 23.8, 13.5 / 24.2
+//   4096 x 14336 (N x K): e4m3 16.9 / 20.8, 18.8 / 20.9, 22.0 / 21.5, 27.1 / 22.8; e2m1 10.6 / 19.7 ... 14.7 / 20.9
+//   16384 x 4096: e4m3 17.9 / 21.6, 16.5 / 21.4, 19.0 / 21.5, 23.5 / 22.7; e2m1 11.9 / 14.8 ... 15.5 / 15.3
+//   2048 x 8192, 1024 x 8192, 4096 x 4096, 8192 x 2048: 0.25 to 0.7 of the tiles' time for every M
+//   28672 x 4096: e4m3 30.0 / 30.0, 29.5 / 29.5, 33.9 / 29.7, 41.4 / 30.6; e2m1 18.6 / 17.2 ... 25.5 / 16.9
+//   32768 x 1024: 1.1 to 2.1 times the tiles' time
+// A group of columns costs its reduction and two barriers whatever K is, so many groups with a short K
+// lose; and with e4m3 operands and more than 32 rows the workgroups' reads of A (every workgroup reads
+// all of it) weigh as much as B once the problem is large.
 bool few_rows_pays(bool fp4, int64_t M, int64_t N, int64_t K, bool have_workspace) {
-  const int64_t cus = device_facts().cu_count;
-  if (M > 64 || N < 8 * cus || K < 4096) return false;
-  const Plan p = plan_for(fp4, M, N);
-  if (M > 32 * p.nt) return false;
-  return fp4 || !have_workspace || M <= 8;
+  (void)have_workspace;
+  if (M > 64 || N < 1024 || K < 2048) return false;
+  if (K < 8192 && N > 16384) return false;
+  if (!fp4 && M > 32 && N * K > ((int64_t)1 << 25)) return false;
+  return true;
 }
 
 int launch_few_rows(bool fp4, const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N,
@@ -250,18 +380,13 @@ int launch_few_rows(bool fp4, const uint8_t* a, const uint8_t* b, const uint8_t*
   int64_t grid = groups;
   if (grid > (int64_t)device_facts().cu_count * per_cu) grid = (int64_t)device_facts().cu_count * per_cu;
   const int stagger = tuning("gemm.few_rows_stagger");
-#define DT_FEW(FP4, MT, NT, WAVES, U)                                                                                    \
-  mx_few_rows_kernel<FP4, MT, NT, WAVES, U><<<(unsigned)grid, WAVES * kWave, 0, stream>>>(a, b, sfa, sfb, (int)M, (int)N, (int)K, \
-                                                                                       lda, ldb, o, ldo, (int)groups, stagger)
-#define DT_FEW_U(FP4, MT, NT, WAVES)                                                      \
-  do {                                                                                    \
-    constexpr int kMaxU = 144 / (2 * (NT + MT) * (FP4 ? 4 : 8));                          \
-    if constexpr (kMaxU >= 4) { if (p.steps == 4) { DT_FEW(FP4, MT, NT, WAVES, 4); break; } } \
-    if constexpr (kMaxU >= 2) { if (p.steps >= 2) { DT_FEW(FP4, MT, NT, WAVES, 2); break; } } \
-    DT_FEW(FP4, MT, NT, WAVES, 1);                                                        \
+#define DT_FEW(FP4, MT, NT, UP) return launch_instance<FP4, MT, NT, UP>(a, b, sfa, sfb, M, N, K, lda, ldb, o, ldo, groups, grid, stagger, stream)
+#define DT_FEW_U(FP4, MT, NT)                                                      \
+  do {                                                                             \
+    if constexpr (MT <= 2 && few_rows_lds_bytes(FP4, MT, 2) < kLdsLimit) { if (p.up == 2) DT_FEW(FP4, MT, NT, 2); } \
+    DT_FEW(FP4, MT, NT, 1);                                                        \
   } while (0)
-#define DT_FEW_W(FP4, MT, NT) do { if (p.waves == 4) DT_FEW_U(FP4, MT, NT, 4); else DT_FEW_U(FP4, MT, NT, 8); } while (0)
-#define DT_FEW_N(FP4, MT) do { if (p.nt == 2) DT_FEW_W(FP4, MT, 2); else DT_FEW_W(FP4, MT, 1); } while (0)
+#define DT_FEW_N(FP4, MT) do { if (p.nt == 2) DT_FEW_U(FP4, MT, 2); else DT_FEW_U(FP4, MT, 1); } while (0)
 #define DT_FEW_M(FP4)                         \
   do {                                        \
     if (mt == 1) DT_FEW_N(FP4, 1);            \
@@ -273,10 +398,9 @@ int launch_few_rows(bool fp4, const uint8_t* a, const uint8_t* b, const uint8_t*
   else DT_FEW_M(false);
 #undef DT_FEW_M
 #undef DT_FEW_N
-#undef DT_FEW_W
 #undef DT_FEW_U
 #undef DT_FEW
-  return launch_status();
+  return DT_ERR_LAUNCH;  // not reached
 }
 
 }  // namespace dt
