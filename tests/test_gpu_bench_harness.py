@@ -36,8 +36,13 @@ def test_harness_timed_table(gpu_device, capsys):
     saved = bench.SHAPES
     bench.SHAPES = [(512, 512), (1, 3232)]
     try:
-        assert bench.main([]) == 0
+        # with the column of the reference's harness that times torch.compile of the eager formulation
+        # (benchmarks/benchmark_saturated_casting.py:122-133)
+        assert bench.main(["--compiled"]) == 0
     finally:
         bench.SHAPES = saved
     text = capsys.readouterr().out
     assert "hip_GBps" in text and "speedup_vs_eager" in text and text.count("bfloat16") == 4
+    header, *table = [line.split() for line in text.strip().splitlines()]
+    col = header.index("compiled_pytorch_time_us")
+    assert len(table) == 4 and all(float(row[col]) > 0 for row in table)
