@@ -302,6 +302,27 @@ def test_mx_gemm_few_rows_kernel(d, cabi, size):
         cabi.set_tuning("gemm.variant", 0)
 
 
+@pytest.mark.parametrize("size", [(16, 256, 20008), (40, 416, 9008), (64, 128, 17000), (3, 1024, 33000)],
+                         ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+@pytest.mark.parametrize("knobs", [dict(tiles=0, steps=0, per_cu=0, stagger=1), dict(tiles=1, steps=1, per_cu=1, stagger=1),
+                                   dict(tiles=2, steps=2, per_cu=1, stagger=0)], ids=lambda k: "-".join(f"{a}{b}" for a, b in k.items()))
+def test_mx_gemm_few_rows_kernel_walks_many_column_groups(d, cabi, size, knobs):
+    """more groups of columns than the grid has workgroups: a workgroup then takes several groups in turn, with
+    the first batch of the next one already on its way while it adds up and stores the one in hand (the sums
+    are parked in the LDS set that has just been used up); every launch shape, with and without the staggered
+    walk along K; the exact product, and the same bits on a second call"""
+    cabi.set_tuning("gemm.variant", 9)
+    for k, v in knobs.items():
+        cabi.set_tuning("gemm.few_rows_" + k, v)
+    try:
+        out, _ = _check_gemm(d, *size, 2500 + size[0], "randn")
+        assert torch.equal(_check_gemm(d, *size, 2500 + size[0], "randn")[0], out)
+    finally:
+        cabi.set_tuning("gemm.variant", 0)
+        for k, v in dict(tiles=0, steps=0, per_cu=0, stagger=1).items():
+            cabi.set_tuning("gemm.few_rows_" + k, v)
+
+
 def test_mx_gemm_few_rows_kernel_is_the_default_and_respects_strides(d, cabi):
     """with enough columns the library takes that kernel by itself; operands and output that are slices of
     wider tensors give the same bits, loads stay inside the rows (poisoned neighbours) and nothing is
