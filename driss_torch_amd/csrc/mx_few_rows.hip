@@ -48,6 +48,8 @@ constexpr int kFewWaves = 8;
 // The value arrives later: nothing may look at it before wait_loads.
 __device__ __forceinline__ v4i load16_async(uint32_t lane_off, const uint8_t* wave_base) {
   v4i r;
+  // (no streaming hint: the two pieces of a lane are the two halves of one line, and with the hint the
+  // second asks memory again: 16 x 8192 x 8192 e4m3 17.6 against 16.4 us)
   asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(lane_off), "s"(wave_base) : "memory");
   return r;
 }
