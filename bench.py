@@ -640,8 +640,9 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False, phases=None):
         bound_ = [bind(cabi, lambda bq=bq, sq=sq: fn(a_q, bq, sa_q, sq, o_)) for bq, sq in sets_]
         us_ = time_launches(lambda i: bound_[i](), ns_, max(50, K // 2), 20)
         hot_ = time_launches(lambda i: bound_[0](), 1, max(50, K // 2), 20)
-        rows.append({"kernel": kernel, "workload": f"{m_rows}x{N}x{Kd} {'e2m1' if fp4 else 'e4m3'} (few rows: B straight from memory into the "
-                     "MFMA's registers, A through LDS, K shared between a workgroup's eight waves)", "bound": "hbm", "avg_us": round(us_, 2),
+        rows.append({"kernel": kernel, "workload": f"{m_rows}x{N}x{Kd} {'e2m1' if fp4 else 'e4m3'} (few rows, one pass over B; the library picks "
+                     "the kernel: B straight from memory into the MFMA's registers and A through LDS, or, for e4m3 with more than 32 "
+                     "rows at this size, 128x128 tiles with K shared between workgroups)", "bound": "hbm", "avg_us": round(us_, 2),
                      "achieved_GBs": round(nb / us_ / 1e3, 1), "frac_of_8TBs": round(nb / us_ / 1e3 / HBM_PEAK_GBS, 4),
                      "hot_cache_us": round(hot_, 2), "algorithmic_bytes": nb, "buffer_sets": ns_})
         del sets_, bound_
