@@ -362,6 +362,9 @@ int launch_instance(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, cons
 
 }  // namespace
 
+// What the kernel takes at all: its 32-bit lane offsets into A's blocked scales span 4 K bytes
+bool few_rows_fits(int64_t M, int64_t K) { return M <= 64 && K <= ((int64_t)1 << 29); }
+
 // Where the kernel above beats the 128 x 128 tiles that share K through a workspace (measured on MI355X,
 // us, B rotated through enough buffers that it comes from HBM; few rows / tiles):
 //   8192 x 8192:  e4m3 M = 8 16.9 / 19.6, 16 16.4 / 19.5, 32 18.8 / 20.0, 64 22.3 / 21.6; e2m1 10.7 / 23.7, 10.9 / 23.7, 12.2 / 23.8, 13.5 / 24.2
@@ -375,7 +378,8 @@ int launch_instance(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, cons
 // all of it) weigh as much as B once the problem is large.
 bool few_rows_pays(bool fp4, int64_t M, int64_t N, int64_t K, bool have_workspace) {
   (void)have_workspace;
-  if (M > 64 || N < 1024 || K < 2048) return false;
+  if (!few_rows_fits(M, K)) return false;
+  if (N < 1024 || K < 2048) return false;
   if (K < 8192 && N > 16384) return false;
   if (!fp4 && M > 32 && N * K > ((int64_t)1 << 25)) return false;
   return true;

@@ -6,6 +6,9 @@
 
 namespace dt {
 
+// Can the kernel for few rows take the problem at all (M <= 64 and a K its 32-bit offsets span)?
+bool few_rows_fits(int64_t M, int64_t K);
+
 // Does the kernel for few rows beat the tiles for this problem?  (fp4: e2m1 operands; K counts elements.)
 bool few_rows_pays(bool fp4, int64_t M, int64_t N, int64_t K, bool have_workspace);
 

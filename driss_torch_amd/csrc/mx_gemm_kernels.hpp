@@ -887,7 +887,7 @@ int mx_gemm(const void* a, const void* b, const uint8_t* sfa, const uint8_t* sfb
   const uint8_t* B = static_cast<const uint8_t*>(b);
   hipStream_t s = as_hip(stream);
   const int variant = tuning("gemm.variant");
-  if ((variant == 9 && M <= 64) || (variant == 0 && few_rows_pays(FP4, M, N, K, workspace != nullptr)))
+  if ((variant == 9 && few_rows_fits(M, K)) || (variant == 0 && few_rows_pays(FP4, M, N, K, workspace != nullptr)))
     return launch_few_rows(FP4, A, B, sfa, sfb, M, N, K, lda, ldb, out, ldo, s);
   const int64_t tiles256 = ceil_div(M, 256) * ceil_div(N, 256);
   const bool big = variant == 2 || variant == 7 || (variant == 0 && tiles256 >= device_facts().cu_count / 2);
