@@ -350,8 +350,10 @@ int launch_instance(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, cons
     (void)hipGetDevice(&dev);
     const bool tracked = dev >= 0 && dev < 16;
     if (!tracked || !allowed[dev].load(std::memory_order_relaxed)) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds) != hipSuccess)
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds) != hipSuccess) {
+        (void)hipGetLastError();  // reported here; the next HIP call must not see it again
         return DT_ERR_LAUNCH;
+      }
       if (tracked) allowed[dev].store(true, std::memory_order_relaxed);
     }
   }
