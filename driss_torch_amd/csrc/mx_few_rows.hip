@@ -7,7 +7,12 @@
 //
 // B goes straight from memory into the registers the MFMA takes: a lane's part of an operand is two
 // 16-byte pieces of one row, 64 bytes apart, and the four lanes that share a row read 64 contiguous bytes
-// of it per load instruction; the E8M0 byte of a lane is one byte of the blocked scale buffer.
+// of it per load instruction.  B's E8M0 bytes: a batch needs one scale word (the four K-blocks of a step)
+// per row, step and tile; one load instruction fetches four of those words, one per group of 16 lanes, and
+// a lane permute hands each lane the word of its row, of which it takes its K-block's byte (a byte load
+// per lane and word, four times as many load instructions, cost 1.0-1.6 us of a launch at 8192 x 8192:
+// measured by leaving them out; this way 16 x 8192 x 8192 e4m3 takes 16.6 against 16.85 us with B from
+// memory and 12.9 against 13.6 us with B in the memory-side cache, e2m1 9.85 against 10.2 and 7.65 against 8.7).
 //
 // A comes out of the L2 (every workgroup reads all of A: M x K bytes, a few hundred KiB), and how it is
 // asked for matters more than B's stream: loaded the way B is, every load instruction asks the L2 for 16
@@ -53,9 +58,9 @@ __device__ __forceinline__ v4i load16_async(uint32_t lane_off, const uint8_t* wa
   asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(lane_off), "s"(wave_base) : "memory");
   return r;
 }
-__device__ __forceinline__ int load_byte_async(uint32_t lane_off, const uint8_t* wave_base) {
+__device__ __forceinline__ int load_word_async(uint32_t lane_off, const uint8_t* wave_base) {
   int r;
-  asm volatile("global_load_ubyte %0, %1, %2" : "=v"(r) : "v"(lane_off), "s"(wave_base) : "memory");
+  asm volatile("global_load_dword %0, %1, %2" : "=v"(r) : "v"(lane_off), "s"(wave_base) : "memory");
   return r;
 }
 // 16 bytes per lane from memory into LDS at lds_addr + 16 * lane, without a register in between
@@ -82,8 +87,13 @@ __global__ __launch_bounds__(kFewWaves* kWave) void mx_few_rows_kernel(const uin
   constexpr int kScaleLoads = (UP * KC + 1) / 2;  // of 1 KiB = two scale chunks
   constexpr int kSetBytes = kPanel + kScaleLoads * 1024, kWaveBytes = 2 * kSetBytes;
   static_assert(MT * NT * 1024 <= kPanel, "a wave parks its sums in the set it has just used up");
+  // B's scale words of a batch: one per (step, chunk of the step, 16-column tile), number (u * KC + c) * NT + j.
+  // One load instruction fetches four of them, one per group of 16 lanes (lane group g' of instruction i
+  // has word 4 i + g' for the 16 rows of that tile), and the lanes that need a word take it from there with
+  // a lane permute: a fourth of the load instructions that a byte per lane and word would be.
+  constexpr int kBWords = UP * KC * NT, kBWordLoads = (kBWords + 3) / 4;
   // loads of a batch, in the order they are issued
-  constexpr int kLoadsPerBatch = UP * NT * 2 + UP * NT * KC + UP * MT * 2 + kScaleLoads;
+  constexpr int kLoadsPerBatch = UP * NT * 2 + kBWordLoads + UP * MT * 2 + kScaleLoads;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x / kWave);
@@ -112,7 +122,17 @@ __global__ __launch_bounds__(kFewWaves* kWave) void mx_few_rows_kernel(const uin
   // A's fragments in LDS: row l16 of a tile = group l16 / 8, row l16 % 8; logical chunks g and 4 + g
   const uint32_t frag_lo = (l16 >> 3) * 1024 + (l16 & 7) * 128 + ((g ^ (l16 & 7)) << 4), frag_hi = frag_lo ^ 64u;
   // a row's scale word inside a 512-byte chunk of 128 rows; the lane's own byte is K-block g
-  auto scale_offset = [&](int row) { return (uint32_t)((row & 31) * 16 + ((row & 127) >> 5) * 4 + g); };
+  auto scale_word_offset = [&](int row) { return (uint32_t)((row & 31) * 16 + ((row & 127) >> 5) * 4); };
+  auto scale_offset = [&](int row) { return scale_word_offset(row) + (uint32_t)g; };
+  // which of B's scale words this lane fetches with load instruction i (clamped to the last one: fetched twice, used once)
+  int bw_u[kBWordLoads], bw_c[kBWordLoads], bw_j[kBWordLoads];
+#pragma unroll
+  for (int i = 0; i < kBWordLoads; ++i) {
+    const int n = 4 * i + g < kBWords ? 4 * i + g : kBWords - 1;
+    bw_j[i] = n % NT;
+    bw_c[i] = (n / NT) % KC;
+    bw_u[i] = n / (NT * KC);
+  }
   uint32_t osa[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) osa[t] = scale_offset(t * 16 + l16 < M ? t * 16 + l16 : M - 1);
@@ -122,7 +142,7 @@ __global__ __launch_bounds__(kFewWaves* kWave) void mx_few_rows_kernel(const uin
   // what of B depends on the column group
   struct Group {
     const uint8_t *b0, *sb0;
-    uint32_t ob[NT], osb[NT];
+    uint32_t ob[NT], osb[kBWordLoads];  // osb: the lane's scale word of load i inside its chunk
   };
   // Which group of columns a workgroup takes in a round of the grid.  Neighbouring groups share the 128-row
   // chunks of B's blocked scales (four groups of 32 columns per chunk), and workgroup b runs on XCD b % 8:
@@ -142,13 +162,17 @@ __global__ __launch_bounds__(kFewWaves* kWave) void mx_few_rows_kernel(const uin
     for (int j = 0; j < NT; ++j) {
       const int brow = n0 + j * 16 + l16 < N ? n0 + j * 16 + l16 : N - 1;  // rows past the edge re-read the last one; never stored
       q.ob[j] = (uint32_t)(brow - n0) * (uint32_t)ldb;
-      q.osb[j] = scale_offset(brow);
+    }
+#pragma unroll
+    for (int i = 0; i < kBWordLoads; ++i) {
+      const int brow = n0 + bw_j[i] * 16 + l16 < N ? n0 + bw_j[i] * 16 + l16 : N - 1;
+      q.osb[i] = scale_word_offset(brow);
     }
     return q;
   };
   struct Batch {
     v4i blo[NT][UP], bhi[NT][UP];
-    int sb[NT][UP][KC];
+    int sbw[kBWordLoads];
   };
   // Everything a batch needs is sent for here: kLoadsPerBatch instructions whatever the batch (a step
   // past the last one reads the last one again and counts as nothing, see consume)
@@ -164,19 +188,18 @@ __global__ __launch_bounds__(kFewWaves* kWave) void mx_few_rows_kernel(const uin
         w.blo[j][u] = load16_async(q.ob[j] + ((tail && !lo_in_tail) ? 0u : (uint32_t)g * 16u), bk);
         w.bhi[j][u] = load16_async(q.ob[j] + ((tail && !hi_in_tail) ? 0u : 64u + (uint32_t)g * 16u), bk);
       }
-#pragma unroll
-      for (int c = 0; c < KC; ++c) {
-        const int kc = p * KC + c < k_chunks ? p * KC + c : k_chunks - 1;
-        const uint8_t* const sbk = q.sb0 + (int64_t)kc * 512;
-#pragma unroll
-        for (int j = 0; j < NT; ++j) w.sb[j][u][c] = load_byte_async(q.osb[j], sbk);
-      }
       const uint8_t* const ak = a + (int64_t)p * 128;
 #pragma unroll
       for (int t = 0; t < MT; ++t)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
           load16_to_lds_async(lds_set + ((u * MT + t) * 2 + h) * 1024, oa[t][h] - (tail ? a_tail_adj : 0u), ak);
+    }
+#pragma unroll
+    for (int i = 0; i < kBWordLoads; ++i) {  // (the chunk's offset is a lane's own here: below 4 K bytes, which the host has bounded)
+      const int p = first_step + bw_u[i] < p_steps ? first_step + bw_u[i] : p_steps - 1;
+      const int kc = p * KC + bw_c[i] < k_chunks ? p * KC + bw_c[i] : k_chunks - 1;
+      w.sbw[i] = load_word_async((uint32_t)kc * 512u + q.osb[i], q.sb0);
     }
     // A's scale chunks of the batch are neighbours in the blocked buffer: 1 KiB = two chunks per instruction
     const int c0 = first_step * KC;
@@ -201,8 +224,10 @@ __global__ __launch_bounds__(kFewWaves* kWave) void mx_few_rows_kernel(const uin
 #pragma unroll
       for (int j = 0; j < NT; ++j) {  // from here on the loaded values may be looked at
         asm volatile("" : "+v"(w.blo[j][u]), "+v"(w.bhi[j][u]));
+      }
+      if (u == 0) {
 #pragma unroll
-        for (int c = 0; c < KC; ++c) asm volatile("" : "+v"(w.sb[j][u][c]));
+        for (int i = 0; i < kBWordLoads; ++i) asm volatile("" : "+v"(w.sbw[i]));
       }
       // elements of K from this step on; the lane's K-block of MFMA c starts 128 c + 32 g elements in
       const int left = K - (first_step + u) * (FP4 ? 256 : 128);
@@ -214,7 +239,10 @@ __global__ __launch_bounds__(kFewWaves* kWave) void mx_few_rows_kernel(const uin
         for (int t = 0; t < MT; ++t) sa[t] = valid ? (int)set_lds[kPanel + (u * KC + c) * 512 + osa[t]] : 0;
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
-          const int sb = valid ? w.sb[j][u][c] : 0;
+          // the tile's scale words sit in lane group n % 4 of load n / 4; this lane's K-block is byte g of its row's
+          const int n = (u * KC + c) * NT + j;
+          const int word = __builtin_amdgcn_ds_bpermute(((n % 4) * 16 + l16) * 4, w.sbw[n / 4]);
+          const int sb = valid ? (int)__builtin_amdgcn_ubfe((uint32_t)word, (uint32_t)g * 8u, 8u) : 0;
           const v8i vb = FP4 ? __builtin_shufflevector(c == 0 ? w.blo[j][u] : w.bhi[j][u], v4i{0, 0, 0, 0}, 0, 1, 2, 3, 4, 5, 6, 7)
                              : __builtin_shufflevector(w.blo[j][u], w.bhi[j][u], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
