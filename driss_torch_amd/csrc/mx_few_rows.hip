@@ -397,12 +397,12 @@ bool few_rows_fits(int64_t M, int64_t K) { return M <= 64 && K <= ((int64_t)1 <<
 
 // Where the kernel above beats the 128 x 128 tiles that share K through a workspace (measured on MI355X,
 // us, B rotated through enough buffers that it comes from HBM; few rows / tiles):
-//   8192 x 8192:  e4m3 M = 8 16.9 / 19.6, 16 16.4 / 19.5, 32 18.8 / 20.0, 64 22.3 / 21.6; e2m1 10.7 / 23.7, 10.9 / 23.7, 12.2 / 23.8, 13.5 / 24.2
-//   4096 x 14336 (N x K): e4m3 16.9 / 20.8, 18.8 / 20.9, 22.0 / 21.5, 27.1 / 22.8; e2m1 10.6 / 19.7 ... 14.7 / 20.9
-//   16384 x 4096: e4m3 17.9 / 21.6, 16.5 / 21.4, 19.0 / 21.5, 23.5 / 22.7; e2m1 11.9 / 14.8 ... 15.5 / 15.3
+//   8192 x 8192:  e4m3 M = 8 17.1 / 19.7, 16 16.4 / 20.0, 32 18.1 / 20.5, 64 21.7 / 21.8; e2m1 10.1 / 21.8, 10.5 / 21.9, 11.6 / 22.0, 13.0 / 22.3
+//   4096 x 14336 (N x K): e4m3 16.8 / 20.9, 18.5 / 21.3, 22.0 / 21.6, 26.9 / 23.0; e2m1 9.9 / 18.1 ... 14.3 / 19.4
+//   16384 x 4096: e4m3 17.2 / 20.2, 16.0 / 20.3, 18.9 / 20.6, 23.9 / 22.0; e2m1 11.1 / 14.4 ... 14.1 / 14.3
 //   2048 x 8192, 1024 x 8192, 4096 x 4096, 8192 x 2048: 0.25 to 0.7 of the tiles' time for every M
-//   28672 x 4096: e4m3 30.0 / 30.0, 29.5 / 29.5, 33.9 / 29.7, 41.4 / 30.6; e2m1 18.6 / 17.2 ... 25.5 / 16.9
-//   32768 x 1024: 1.1 to 2.1 times the tiles' time
+//   28672 x 4096: e4m3 28.7 / 29.9, 28.7 / 28.9, 33.3 / 29.1, 41.4 / 30.3; e2m1 17.4 / 16.5 ... 24.3 / 16.8
+//   32768 x 1024: 1.1 to 1.9 times the tiles' time
 // A group of columns costs its reduction and two barriers whatever K is, so many groups with a short K
 // lose; and with e4m3 operands and more than 32 rows the workgroups' reads of A (every workgroup reads
 // all of it) weigh as much as B once the problem is large.
