@@ -74,14 +74,17 @@ __device__ __forceinline__ void wait_loads() {
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-template <bool FP4, int MT, int NT, int UP>
+// MH: A's rows in halves of a 16-row tile (8 rows, one LDS-DMA instruction per step); the second half of
+// the last tile is not fetched when no row of A lies in it (its sums are never stored)
+template <bool FP4, int MH, int NT, int UP>
 __global__ __launch_bounds__(kFewWaves* kWave) void mx_few_rows_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                                                                      const uint8_t* __restrict__ sfa, const uint8_t* __restrict__ sfb,
                                                                      int M, int N, int K, int64_t lda, int64_t ldb,
                                                                      uint16_t* __restrict__ out, int64_t ldo, int groups, int stagger) {
   constexpr int WAVES = kFewWaves;
+  constexpr int MT = (MH + 1) / 2;
   constexpr int KC = FP4 ? 2 : 1;  // MFMAs, and blocked scale chunks, per panel step of 128 bytes of a row
-  static_assert(MT >= 1 && MT <= 4 && NT >= 1 && NT <= 2 && UP >= 1, "at most 64 rows of A, 32 columns per group");
+  static_assert(MH >= 1 && MH <= 8 && NT >= 1 && NT <= 2 && UP >= 1, "at most 64 rows of A, 32 columns per group");
   // LDS of a wave: two sets of [A rows of a batch: step, tile, half of 8 rows, 8 rows x 128 B][A scale chunks of the batch]
   constexpr int kPanel = UP * MT * 2048;
   constexpr int kScaleLoads = (UP * KC + 1) / 2;  // of 1 KiB = two scale chunks
@@ -93,7 +96,7 @@ __global__ __launch_bounds__(kFewWaves* kWave) void mx_few_rows_kernel(const uin
   // a lane permute: a fourth of the load instructions that a byte per lane and word would be.
   constexpr int kBWords = UP * KC * NT, kBWordLoads = (kBWords + 3) / 4;
   // loads of a batch, in the order they are issued
-  constexpr int kLoadsPerBatch = UP * NT * 2 + kBWordLoads + UP * MT * 2 + kScaleLoads;
+  constexpr int kLoadsPerBatch = UP * NT * 2 + kBWordLoads + UP * MH + kScaleLoads;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x / kWave);
@@ -193,7 +196,7 @@ __global__ __launch_bounds__(kFewWaves* kWave) void mx_few_rows_kernel(const uin
       for (int t = 0; t < MT; ++t)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
-          load16_to_lds_async(lds_set + ((u * MT + t) * 2 + h) * 1024, oa[t][h] - (tail ? a_tail_adj : 0u), ak);
+          if (t * 2 + h < MH) load16_to_lds_async(lds_set + ((u * MT + t) * 2 + h) * 1024, oa[t][h] - (tail ? a_tail_adj : 0u), ak);
     }
 #pragma unroll
     for (int i = 0; i < kBWordLoads; ++i) {  // (the chunk's offset is a lane's own here: below 4 K bytes, which the host has bounded)
@@ -353,10 +356,13 @@ constexpr size_t few_rows_lds_bytes(bool fp4, int mt, int up) {
 }
 constexpr size_t kLdsLimit = 160 * 1024;
 
+// Two tiles per group halve the workgroups' reads of A (every group reads all of it) and win wherever they
+// still give every CU a group (8192 x 8192, us, one tile / two: e4m3 1 row 16.2 / 15.6, 8 rows 16.8 / 15.8,
+// 16 rows 18.3 / 16.5, 56 rows 28.9 / 20.9; e2m1 1 row 10.9 / 9.4, 56 rows 16.5 / 12.2).
 Plan plan_for(bool fp4, int64_t M, int64_t N) {
   Plan p;
   const int tiles = tuning("gemm.few_rows_tiles");
-  p.nt = tiles ? (tiles == 2 ? 2 : 1) : (N >= 32 * (int64_t)device_facts().cu_count && (fp4 || M > 8) ? 2 : 1);
+  p.nt = tiles ? (tiles == 2 ? 2 : 1) : (N >= 32 * (int64_t)device_facts().cu_count ? 2 : 1);
   const int mt = (int)((M + 15) / 16);
   int up = tuning("gemm.few_rows_steps");
   if (up != 1 && up != 2) up = mt == 1 ? 2 : 1;
@@ -365,13 +371,13 @@ Plan plan_for(bool fp4, int64_t M, int64_t N) {
   return p;
 }
 
-template <bool FP4, int MT, int NT, int UP>
+template <bool FP4, int MH, int NT, int UP>
 int launch_instance(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb, int64_t M, int64_t N, int64_t K,
                     int64_t lda, int64_t ldb, uint16_t* out, int64_t ldo, int64_t groups, int64_t grid, int stagger,
                     hipStream_t stream) {
-  constexpr size_t kLds = few_rows_lds_bytes(FP4, MT, UP);
+  constexpr size_t kLds = few_rows_lds_bytes(FP4, (MH + 1) / 2, UP);
   static_assert(kLds <= kLdsLimit, "two sets per wave fit the CU's LDS");
-  auto kernel = mx_few_rows_kernel<FP4, MT, NT, UP>;
+  auto kernel = mx_few_rows_kernel<FP4, MH, NT, UP>;
   if (kLds > 64 * 1024) {  // once per instantiation and device
     static std::atomic<bool> allowed[16];
     int dev = 0;
@@ -397,11 +403,11 @@ bool few_rows_fits(int64_t M, int64_t K) { return M <= 64 && K <= ((int64_t)1 <<
 
 // Where the kernel above beats the 128 x 128 tiles that share K through a workspace (measured on MI355X,
 // us, B rotated through enough buffers that it comes from HBM; few rows / tiles):
-//   8192 x 8192:  e4m3 M = 8 17.1 / 19.7, 16 16.4 / 20.0, 32 18.1 / 20.5, 64 21.7 / 21.8; e2m1 10.1 / 21.8, 10.5 / 21.9, 11.6 / 22.0, 13.0 / 22.3
-//   4096 x 14336 (N x K): e4m3 16.8 / 20.9, 18.5 / 21.3, 22.0 / 21.6, 26.9 / 23.0; e2m1 9.9 / 18.1 ... 14.3 / 19.4
-//   16384 x 4096: e4m3 17.2 / 20.2, 16.0 / 20.3, 18.9 / 20.6, 23.9 / 22.0; e2m1 11.1 / 14.4 ... 14.1 / 14.3
+//   8192 x 8192:  e4m3 M = 8 15.7 / 20.7, 16 16.4 / 20.0, 32 18.1 / 20.5, 64 21.7 / 21.8; e2m1 10.1 / 21.8, 10.5 / 21.9, 11.6 / 22.0, 13.0 / 22.3
+//   4096 x 14336 (N x K): e4m3 16.5 / 20.8, 18.5 / 21.3, 22.0 / 21.6, 26.9 / 23.0; e2m1 9.9 / 18.1 ... 14.3 / 19.4
+//   16384 x 4096: e4m3 15.3 / 20.3, 16.0 / 20.3, 18.9 / 20.6, 23.9 / 22.0; e2m1 11.1 / 14.4 ... 14.1 / 14.3
 //   2048 x 8192, 1024 x 8192, 4096 x 4096, 8192 x 2048: 0.25 to 0.7 of the tiles' time for every M
-//   28672 x 4096: e4m3 28.7 / 29.9, 28.7 / 28.9, 33.3 / 29.1, 41.4 / 30.3; e2m1 17.4 / 16.5 ... 24.3 / 16.8
+//   28672 x 4096: e4m3 27.2 / 31.1, 28.7 / 28.9, 33.3 / 29.1, 41.4 / 30.3; e2m1 17.4 / 16.5 ... 24.3 / 16.8
 //   32768 x 1024: 1.1 to 1.9 times the tiles' time
 // A group of columns costs its reduction and two barriers whatever K is, so many groups with a short K
 // lose; and with e4m3 operands and more than 32 rows the workgroups' reads of A (every workgroup reads
@@ -419,26 +425,32 @@ int launch_few_rows(bool fp4, const uint8_t* a, const uint8_t* b, const uint8_t*
                     int64_t K, int64_t lda, int64_t ldb, void* out, int64_t ldo, hipStream_t stream) {
   uint16_t* o = static_cast<uint16_t*>(out);
   const Plan p = plan_for(fp4, M, N);
-  const int mt = (int)((M + 15) / 16);
+  const int mh = (int)((M + 7) / 8);  // halves of 16-row tiles that hold rows of A
   const int64_t groups = ceil_div(N, (int64_t)16 * p.nt);
   int per_cu = tuning("gemm.few_rows_per_cu");
   if (per_cu < 1) per_cu = 2;
   int64_t grid = groups;
   if (grid > (int64_t)device_facts().cu_count * per_cu) grid = (int64_t)device_facts().cu_count * per_cu;
   const int stagger = tuning("gemm.few_rows_stagger");
-#define DT_FEW(FP4, MT, NT, UP) return launch_instance<FP4, MT, NT, UP>(a, b, sfa, sfb, M, N, K, lda, ldb, o, ldo, groups, grid, stagger, stream)
-#define DT_FEW_U(FP4, MT, NT)                                                      \
+#define DT_FEW(FP4, MH, NT, UP) return launch_instance<FP4, MH, NT, UP>(a, b, sfa, sfb, M, N, K, lda, ldb, o, ldo, groups, grid, stagger, stream)
+#define DT_FEW_U(FP4, MH, NT)                                                      \
   do {                                                                             \
-    if constexpr (MT <= 2 && few_rows_lds_bytes(FP4, MT, 2) < kLdsLimit) { if (p.up == 2) DT_FEW(FP4, MT, NT, 2); } \
-    DT_FEW(FP4, MT, NT, 1);                                                        \
+    if constexpr (MH <= 4 && few_rows_lds_bytes(FP4, (MH + 1) / 2, 2) < kLdsLimit) { if (p.up == 2) DT_FEW(FP4, MH, NT, 2); } \
+    DT_FEW(FP4, MH, NT, 1);                                                        \
   } while (0)
-#define DT_FEW_N(FP4, MT) do { if (p.nt == 2) DT_FEW_U(FP4, MT, 2); else DT_FEW_U(FP4, MT, 1); } while (0)
+#define DT_FEW_N(FP4, MH) do { if (p.nt == 2) DT_FEW_U(FP4, MH, 2); else DT_FEW_U(FP4, MH, 1); } while (0)
 #define DT_FEW_M(FP4)                         \
   do {                                        \
-    if (mt == 1) DT_FEW_N(FP4, 1);            \
-    else if (mt == 2) DT_FEW_N(FP4, 2);       \
-    else if (mt == 3) DT_FEW_N(FP4, 3);       \
-    else DT_FEW_N(FP4, 4);                    \
+    switch (mh) {                             \
+      case 1: DT_FEW_N(FP4, 1);               \
+      case 2: DT_FEW_N(FP4, 2);               \
+      case 3: DT_FEW_N(FP4, 3);               \
+      case 4: DT_FEW_N(FP4, 4);               \
+      case 5: DT_FEW_N(FP4, 5);               \
+      case 6: DT_FEW_N(FP4, 6);               \
+      case 7: DT_FEW_N(FP4, 7);               \
+      default: DT_FEW_N(FP4, 8);              \
+    }                                         \
   } while (0)
   if (fp4) DT_FEW_M(true);
   else DT_FEW_M(false);

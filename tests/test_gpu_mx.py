@@ -290,10 +290,11 @@ def test_mx_gemm_ignores_the_padding_of_the_scale_buffers(d, cabi, variant, size
 
 
 @pytest.mark.parametrize("size", [(1, 640, 8), (16, 2048, 256), (17, 96, 2056), (33, 1120, 264), (48, 416, 136), (64, 8192, 512),
-                                  (5, 32, 24), (64, 160, 16)], ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+                                  (5, 32, 24), (64, 160, 16), (8, 416, 264), (9, 288, 40), (24, 1120, 136), (28, 416, 264),
+                                  (40, 2048, 64), (52, 160, 520), (56, 2080, 72)], ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
 def test_mx_gemm_few_rows_kernel(d, cabi, size):
     """the kernel for problems of at most 64 rows (16 columns per workgroup, K shared between its eight
-    waves, operands straight from memory): every count of 16-row tiles, ragged M and N, K with a partly
+    waves, operands straight from memory): every count of 8-row halves of A's tiles, ragged M and N, K with a partly
     filled last 128-element step; forced here for every N, and checked against the exact product"""
     cabi.set_tuning("gemm.variant", 9)
     try:

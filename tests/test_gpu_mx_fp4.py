@@ -89,7 +89,8 @@ def test_mx_fp4_gemm_k_of_any_whole_number_of_blocks(d, cabi, variant, K):
 
 
 @pytest.mark.parametrize("size", [(1, 640, 8), (16, 2048, 256), (17, 96, 2056), (33, 1312, 264), (48, 480, 136), (64, 8192, 512),
-                                  (5, 32, 24), (24, 4128, 4104)], ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
+                                  (5, 32, 24), (24, 4128, 4104), (8, 480, 264), (28, 416, 264), (40, 2048, 64), (52, 160, 520),
+                                  (56, 2080, 72)], ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}")
 def test_mx_fp4_gemm_few_rows_kernel(d, cabi, size):
     """the kernel for problems of at most 64 rows, forced for every N (the last size takes it by default
     too): every count of 16-row tiles, ragged M and N, K with a partly filled last 128-element step"""
