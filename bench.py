@@ -553,6 +553,19 @@ def extra_kernels(torch, cabi, dev, K, W, gemm_only=False, phases=None):
                            torch.empty((nblk,), dtype=torch.uint8, device=dev)),
                 lambda x, dd, sc: cabi.mx_fp4_quantize(x, cabi.SCALE_BLOCKED, dd, sc))
 
+        nblk_c = cabi.lib().dt_blocked_scale_bytes(8192, 256)
+        hbm_row("mx_fp4_quantize_dual (rows + transposed columns from one read)",
+                "bf16 [8192,8192] -> two packed e2m1 payloads + E8M0, blocked scales", 8192 * 8192 * (2 + 2 * (0.5 + 1 / 32)),
+                lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 4096), dtype=torch.uint8, device=dev),
+                           torch.empty((nblk,), dtype=torch.uint8, device=dev), torch.empty((8192, 4096), dtype=torch.uint8, device=dev),
+                           torch.empty((nblk_c,), dtype=torch.uint8, device=dev)),
+                lambda x, dr, sr, dc, sc: cabi.mx_fp4_quantize_dual(x, cabi.SCALE_BLOCKED, (dr, sr, dc, sc)))
+        hbm_row("mx_fp4_quantize cols (transposed out), blocked scales", "bf16 [8192,8192] -> packed e2m1 [8192,4096] + E8M0",
+                8192 * 8192 * (2 + 0.5 + 1 / 32),
+                lambda i: (rnd((8192, 8192), bf16, i), torch.empty((8192, 4096), dtype=torch.uint8, device=dev),
+                           torch.empty((nblk_c,), dtype=torch.uint8, device=dev)),
+                lambda x, dd, sc: cabi.mx_fp4_quantize(x, cabi.SCALE_BLOCKED, dd, sc, 0))
+
     if not gemm_only:
         hbm_rows()
 

@@ -151,6 +151,12 @@ def mx_fp4_quantize(input: Tensor, blocked: bool = False, axis: int = 1) -> Tupl
     return ops.mx_fp4_quantize(input, blocked, axis)
 
 
+def mx_fp4_quantize_dual(input: Tensor, blocked: bool = False) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """Both MXFP4 operands of ``input`` [M, N] from one read: ``(data [M, N/2], scale, data_t [N, M/2],
+    scale_t)``, equal to ``mx_fp4_quantize(input, blocked, 1) + mx_fp4_quantize(input, blocked, 0)``."""
+    return ops.mx_fp4_quantize_dual(input, blocked)
+
+
 def to_blocked(scale: Tensor) -> Tensor:
     """[R, C] E8M0 scale matrix -> flat blocked 128x4 layout (zero padded)."""
     return ops.to_blocked(scale)

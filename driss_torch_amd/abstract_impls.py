@@ -92,6 +92,10 @@ def mx_fp4_quantize_meta(x, blocked, axis):
             torch.empty((nscale,), dtype=torch.float8_e8m0fnu, device=x.device))
 
 
+def mx_fp4_quantize_dual_meta(x, blocked):
+    return mx_fp4_quantize_meta(x, blocked, 1) + mx_fp4_quantize_meta(x, blocked, 0)
+
+
 def to_blocked_meta(scale):
     r, c = scale.shape
     return torch.empty((128 * _ceil_div(r, 128) * 4 * _ceil_div(c, 4),), dtype=scale.dtype, device=scale.device)
@@ -118,6 +122,7 @@ FAKE_IMPLS = {
     "DrissTorch::mx_fp8_quantize_ex": mx_fp8_quantize_ex_meta,
     "DrissTorch::mx_fp8_quantize_dual": mx_fp8_quantize_dual_meta,
     "DrissTorch::mx_fp4_quantize": mx_fp4_quantize_meta,
+    "DrissTorch::mx_fp4_quantize_dual": mx_fp4_quantize_dual_meta,
     "DrissTorch::to_blocked": to_blocked_meta,
     "DrissTorch::mx_fp8_bf16": mx_fp8_bf16_meta,
     "DrissTorch::mx_fp4_bf16": mx_fp4_bf16_meta,

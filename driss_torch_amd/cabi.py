@@ -43,6 +43,7 @@ SIGNATURES = {
     "dt_mx_fp8_quantize": (_i32, [_vp, _i32, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
     "dt_mx_fp8_quantize_dual": (_i32, [_vp, _i32, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "dt_mx_fp4_quantize": (_i32, [_vp, _i32, _i64, _i64, _i32, _i32, _vp, _vp, _vp]),
+    "dt_mx_fp4_quantize_dual": (_i32, [_vp, _i32, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp]),
     "dt_blocked_scale_bytes": (_i64, [_i64, _i64]),
     "dt_to_blocked": (_i32, [_vp, _i64, _i64, _vp, _vp]),
     "dt_mx_fp8_bf16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
@@ -274,6 +275,21 @@ def mx_fp4_quantize(x: torch.Tensor, layout: int = 0, data=None, scale=None, axi
     _check(lib().dt_mx_fp4_quantize(x.data_ptr(), IN_DTYPE[x.dtype], R, Cc, axis, layout, data.data_ptr(), scale.data_ptr(),
                                     _stream()), "dt_mx_fp4_quantize")
     return data, scale
+
+
+def mx_fp4_quantize_dual(x: torch.Tensor, layout: int = SCALE_PLAIN, outs=None):
+    """(data_rows [R, C/2], scale_rows, data_cols_t [C, R/2], scale_cols_t): the axis-1 and the axis-0 MXFP4
+    cast of x from one read of x.  `outs`: the four output tensors, to reuse them."""
+    R, Cc = x.shape
+    if outs is None:
+        n_r = lib().dt_blocked_scale_bytes(R, Cc // 32) if layout == SCALE_BLOCKED else R * (Cc // 32)
+        n_c = lib().dt_blocked_scale_bytes(Cc, R // 32) if layout == SCALE_BLOCKED else Cc * (R // 32)
+        outs = (torch.empty((R, Cc // 2), dtype=torch.uint8, device=x.device), torch.empty((n_r,), dtype=torch.uint8, device=x.device),
+                torch.empty((Cc, R // 2), dtype=torch.uint8, device=x.device), torch.empty((n_c,), dtype=torch.uint8, device=x.device))
+    dr, sr, dc, sc = outs
+    _check(lib().dt_mx_fp4_quantize_dual(x.data_ptr(), IN_DTYPE[x.dtype], R, Cc, layout, dr.data_ptr(), sr.data_ptr(),
+                                         dc.data_ptr(), sc.data_ptr(), _stream()), "dt_mx_fp4_quantize_dual")
+    return dr, sr, dc, sc
 
 
 def to_blocked(scale: torch.Tensor) -> torch.Tensor:

@@ -240,6 +240,21 @@ int launch_mx_fp4(const MxArgs& a) {
 // blocks down the columns, payload transposed: [cols, rows/2], scales [cols, rows/32]
 template <int IN, int LAYOUT>
 int launch_mx_fp4_cols(const MxArgs& a) {
+  // As for MXFP8, the one-read kernel without its row-wise half, on its grid of walking workgroups, for
+  // 16-bit inputs with more tiles than that grid (bf16, us, this / mx_col_t_kernel: 8192 x 8192 33.1 / 33.9,
+  // 16384 x 4096 30.5 / 35.5, 4096 x 16384 31.5 / 31.7; it loses for fp32, 55.4 / 51.9, and for small
+  // tensors, 2048 x 4096 6.6 / 5.9)
+  constexpr int kV = InTraits<IN>::kVec;
+  if constexpr (IN != DT_F32) {
+    const int64_t pipe_grid = (int64_t)tuning("mx.colt_pipe") * device_facts().cu_count;
+    const int64_t dual_tiles = ceil_div(a.rows, (int64_t)kDualRows) * ceil_div(a.cols, (int64_t)(32 * kV));
+    if (a.cols % kV == 0 && tuning("mx.colt_via_dual") && pipe_grid > 0 && dual_tiles > pipe_grid && dual_tiles <= 0x7FFFFFFFll) {
+      const int order = tuning("mx.dual_order") >= 0 ? tuning("mx.dual_order") : (a.rows % (8 * kDualRows) == 0 ? 2 : (a.cols < a.rows ? 1 : 0));
+      mx_dual_kernel<IN, DT_E2M1, LAYOUT, false, true><<<(unsigned)pipe_grid, kBlock, 0, a.stream>>>(
+          a.x, (uint32_t)a.rows, (uint32_t)a.cols, nullptr, nullptr, a.data, a.scale, order);
+      return launch_status();
+    }
+  }
   const int64_t tiles = ceil_div(a.rows, (int64_t)kColTRows) * ceil_div(a.cols, (int64_t)kColTCols);
   if (tiles > 0x7FFFFFFFll) return DT_ERR_INVALID_SHAPE;
   mx_col_t_kernel<IN, DT_E2M1, LAYOUT><<<(unsigned)tiles, kBlock, 0, a.stream>>>(a.x, (uint32_t)a.rows, (uint32_t)a.cols, a.data,
@@ -285,6 +300,58 @@ extern "C" int dt_mx_fp4_quantize(const void* x, int in_dtype, int64_t rows, int
     case DT_BF16: return blocked ? launch_mx_fp4<DT_BF16, DT_SCALE_BLOCKED>(a) : launch_mx_fp4<DT_BF16, DT_SCALE_PLAIN>(a);
     default: return blocked ? launch_mx_fp4<DT_F16, DT_SCALE_BLOCKED>(a) : launch_mx_fp4<DT_F16, DT_SCALE_PLAIN>(a);
   }
+}
+
+namespace {
+// both MXFP4 operands of one tensor from a single read: mx_dual_kernel with the e2m1 output code
+template <int IN, int LAYOUT>
+int launch_dual_fp4(const DualArgs& a) {
+  constexpr int kTileCols = 32 * InTraits<IN>::kVec;
+  if (!aligned(a.data_r, 4) || !aligned(a.data_c, 16) || !aligned(a.scale_r, 4) || !aligned(a.scale_c, 4) ||
+      a.rows >= (1ll << 31) || a.cols >= (1ll << 31))
+    return kNotTaken;
+  const int64_t tiles = ceil_div(a.rows, (int64_t)kDualRows) * ceil_div(a.cols, (int64_t)kTileCols);
+  if (tiles > 0x7FFFFFFFll) return kNotTaken;
+  const int order = tuning("mx.dual_order") >= 0 ? tuning("mx.dual_order")
+                    : a.cols > 2 * a.rows                ? 0
+                    : a.rows % (8 * kDualRows) == 0      ? 2
+                                                         : 1;
+  mx_dual_kernel<IN, DT_E2M1, LAYOUT><<<(unsigned)tiles, kBlock, 0, a.stream>>>(a.x, (uint32_t)a.rows, (uint32_t)a.cols, a.data_r,
+                                                                               a.scale_r, a.data_c, a.scale_c, order);
+  return launch_status();
+}
+template <int IN>
+int launch_dual_fp4_in(const DualArgs& a, int layout) {
+  return layout == DT_SCALE_BLOCKED ? launch_dual_fp4<IN, DT_SCALE_BLOCKED>(a) : launch_dual_fp4<IN, DT_SCALE_PLAIN>(a);
+}
+}  // namespace
+
+extern "C" int dt_mx_fp4_quantize_dual(const void* x, int in_dtype, int64_t rows, int64_t cols, int scale_layout, void* data_rows,
+                                       uint8_t* scale_rows, void* data_cols_t, uint8_t* scale_cols_t, dt_stream_t stream) {
+  if (in_dtype != DT_F32 && in_dtype != DT_BF16 && in_dtype != DT_F16) return DT_ERR_INVALID_DTYPE;
+  if (scale_layout != DT_SCALE_PLAIN && scale_layout != DT_SCALE_BLOCKED) return DT_ERR_INVALID_MODE;
+  if (rows < 0 || cols < 0 || rows % 32 != 0 || cols % 32 != 0) return DT_ERR_INVALID_SHAPE;
+  if (rows == 0 || cols == 0) return DT_OK;
+  if (!x || !data_rows || !scale_rows || !data_cols_t || !scale_cols_t) return DT_ERR_NULL_POINTER;
+  if (!dt::aligned(x, in_dtype == DT_F32 ? 4 : 2)) return DT_ERR_MISALIGNED;
+  hipStream_t s = dt::as_hip(stream);
+  DualArgs a{x, rows, cols, static_cast<uint8_t*>(data_rows), scale_rows, static_cast<uint8_t*>(data_cols_t), scale_cols_t, s};
+  if (dt::tuning("mx.dual") != 0) {
+    if (scale_layout == DT_SCALE_BLOCKED) {
+      if (int st = zero_blocked_padding(scale_rows, rows, cols / 32, s)) return st;
+      if (int st = zero_blocked_padding(scale_cols_t, cols, rows / 32, s)) return st;
+    }
+    int st;
+    switch (in_dtype) {
+      case DT_F32: st = launch_dual_fp4_in<DT_F32>(a, scale_layout); break;
+      case DT_BF16: st = launch_dual_fp4_in<DT_BF16>(a, scale_layout); break;
+      default: st = launch_dual_fp4_in<DT_F16>(a, scale_layout); break;
+    }
+    if (st != kNotTaken) return st;
+  }
+  // two passes over x
+  if (int st = dt_mx_fp4_quantize(x, in_dtype, rows, cols, 1, scale_layout, data_rows, scale_rows, stream)) return st;
+  return dt_mx_fp4_quantize(x, in_dtype, rows, cols, 0, scale_layout, data_cols_t, scale_cols_t, stream);
 }
 
 extern "C" int dt_to_blocked(const uint8_t* scale, int64_t R, int64_t C, uint8_t* out, dt_stream_t stream) {

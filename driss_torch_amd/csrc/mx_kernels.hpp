@@ -537,6 +537,8 @@ __global__ __launch_bounds__(kBlock) void mx_col_t_kernel(const void* __restrict
 // with bits 4..6 of the column so that the 16 lanes of one write phase (columns kV apart) fall
 // on 16 different bank groups.
 constexpr int kDualRows = 128, kDualPitch = 144;
+// (e2m1 output: a column's 128 rows are 64 bytes; pitch 80, the chunk index XORed with bits 4..5 of the column)
+constexpr int kDualPitch4 = 80;
 
 __device__ __forceinline__ uint32_t other_half_max_u32(uint32_t v) {
   const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);  // [0]: lower half's value, [1]: upper half's
@@ -666,6 +668,26 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
 #pragma unroll
   for (int c = 0; c < kV; ++c) {
     const MxScale<OUT> s = mx_scale_from_absbits<OUT>(cm[c]);
+    if constexpr (OUT == DT_E2M1) {
+      // two rows of x per byte: the lane's 16 rows of a column are 8 bytes, the half h of the wave's
+      // 16-byte chunk w of that column's 64 (byte j of a word = rows 8 q + 2 j in the low nibble, + 1 in the high)
+      uint32_t r2[2];
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        uint32_t r = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int i = 8 * q + 2 * j;
+          if constexpr (IN == DT_F32) r = cvt_fp4_pair32(r, word(i, c), word(i + 1, c), s.scale, j);
+          else r = cvt_fp4_pair16<IN>(r, gather_halves(c & 1, word(i, c), word(i + 1, c)), s.scale, j);
+        }
+        r2[q] = s.nan ? 0x77777777u : r;
+      }
+      const uint32_t col = (uint32_t)(c8 * kV + c);
+      *reinterpret_cast<u32x2*>(tile + col * kDualPitch4 + ((((uint32_t)w) ^ ((col >> 4) & 3u)) << 4) + h * 8) = u32x2{r2[0], r2[1]};
+      if (h == 0) reinterpret_cast<uint8_t*>(ctile)[col * 4 + w] = (uint8_t)(active ? s.byte : 0u);
+      continue;
+    }
     uint32_t r[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
@@ -691,7 +713,17 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
     const MxScale<OUT> s = mx_scale_from_absbits<OUT>(m);
     rb[i / 4] |= s.byte << (8 * (i % 4));
     if (active) {
-      if constexpr (IN == DT_F32) {
+      if constexpr (OUT == DT_E2M1) {
+        // two columns per byte: a lane's kV columns leave as kV / 2 bytes of the row's cols / 2
+        uint8_t* const d4 = data_r + (uint64_t)(row0 + i) * (cols / 2) + col0 / 2;
+        if constexpr (IN == DT_F32) {
+          const uint32_t r = cvt_fp4_4x32(v[i], s.scale);
+          *reinterpret_cast<uint16_t*>(d4) = (uint16_t)(s.nan ? 0x7777u : r);
+        } else {
+          const uint32_t r = cvt_fp4_8x16<IN>(v[i], s.scale);
+          st_stream(reinterpret_cast<uint32_t*>(d4), s.nan ? 0x77777777u : r);
+        }
+      } else if constexpr (IN == DT_F32) {
         const uint32_t r = cvt_scaled_4x32<OUT>(v[i].x, v[i].y, v[i].z, v[i].w, s.scale);
         st_stream(reinterpret_cast<uint32_t*>(drow + (uint64_t)i * cols), s.nan ? 0x7F7F7F7Fu : r);
       } else {
@@ -709,6 +741,16 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
 
   // ---- transposed payload: kTileCols output rows (columns of x) x 8 chunks of 16 bytes
   const uint32_t trow0 = tr * kDualRows, tcol0 = tc * kTileCols;
+  if constexpr (OUT == DT_E2M1) {  // 4 chunks of 16 bytes (32 rows of x each) per output row of rows / 2 bytes
+#pragma unroll
+    for (int i = 0; i < kTileCols * 4 / kBlock; ++i) {
+      const uint32_t id = tid + i * kBlock, r = id >> 2, q = id & 3;
+      if (tcol0 + r < cols && trow0 + q * 32 < rows) {
+        const u32x4 o = *reinterpret_cast<const u32x4*>(tile + r * kDualPitch4 + ((q ^ ((r >> 4) & 3u)) << 4));
+        *reinterpret_cast<u32x4*>(data_c + (uint64_t)(tcol0 + r) * (rows / 2) + trow0 / 2 + q * 16) = o;
+      }
+    }
+  } else {
 #pragma unroll
   for (int i = 0; i < kTileCols * 8 / kBlock; ++i) {
     const uint32_t id = tid + i * kBlock, r = id >> 3, q = id & 7;
@@ -718,6 +760,7 @@ __global__ __launch_bounds__(kBlock) void mx_dual_kernel(const void* __restrict_
       // write-back from L2 beats streaming stores (8192 x 8192 bf16: 47.4 vs 54.1 us for the kernel)
       *reinterpret_cast<u32x4*>(data_c + (uint64_t)(tcol0 + r) * rows + trow0 + q * 16) = o;
     }
+  }
   }
   // ---- column-block scales [cols, rows/32]: 4 bytes per column of this tile
   const uint32_t RB = rows / 32, rb0 = tr * 4;

@@ -325,6 +325,32 @@ std::tuple<Tensor, Tensor> mx_fp4_quantize(const Tensor& input, bool blocked, in
   return {data, scale};
 }
 
+// Both MXFP4 operands of one tensor from a single read: mx_fp4_quantize(input, blocked, 1) and
+// mx_fp4_quantize(input, blocked, 0).  No counterpart op in the reference (see mx_fp4_quantize).
+std::tuple<Tensor, Tensor, Tensor, Tensor> mx_fp4_quantize_dual(const Tensor& input, bool blocked) {
+  TORCH_CHECK(input.is_cuda(), "Input tensor must be a CUDA tensor");
+  TORCH_CHECK(input.is_contiguous(), "Input tensor must be contiguous");
+  TORCH_CHECK(input.scalar_type() == at::kHalf || input.scalar_type() == at::kFloat ||
+                  input.scalar_type() == at::kBFloat16,
+              "Input tensor must be float, half, or bfloat16");
+  TORCH_CHECK(input.dim() == 2, "Only support 2d tensor for now");
+  const int64_t m = input.size(0), n = input.size(1);
+  TORCH_CHECK(m % 32 == 0 && n % 32 == 0, "Need block shape to evenly divide the input tensor for now");
+  Ctx ctx(input);
+  const auto u8 = input.options().dtype(at::kByte);
+  const auto e8 = input.options().dtype(at::kFloat8_e8m0fnu);
+  Tensor data_r = at::empty({m, n / 2}, u8), data_c = at::empty({n, m / 2}, u8);
+  Tensor scale_r = at::empty({blocked ? dt_blocked_scale_bytes(m, n / 32) : m * (n / 32)}, e8);
+  Tensor scale_c = at::empty({blocked ? dt_blocked_scale_bytes(n, m / 32) : n * (m / 32)}, e8);
+  if (input.numel() == 0) return {data_r, scale_r, data_c, scale_c};
+  TORCH_CHECK(reinterpret_cast<std::uintptr_t>(input.data_ptr()) % 16 == 0, "Input tensor must be 16-byte aligned");
+  check_status(dt_mx_fp4_quantize_dual(input.data_ptr(), in_code(input), m, n, blocked ? DT_SCALE_BLOCKED : DT_SCALE_PLAIN,
+                                       data_r.data_ptr(), static_cast<uint8_t*>(scale_r.data_ptr()), data_c.data_ptr(),
+                                       static_cast<uint8_t*>(scale_c.data_ptr()), ctx.stream),
+               "mx_fp4_quantize_dual");
+  return {data_r, scale_r, data_c, scale_c};
+}
+
 // ------------------------------------------------------------------------ mx_fp8_bf16
 // src/mx_fp8_bf16.cu:168-241
 Tensor mx_fp8_bf16(Tensor a, Tensor b, Tensor a_scale, Tensor b_scale) {
@@ -456,6 +482,8 @@ TORCH_LIBRARY(DrissTorch, m) {
   m.impl("mx_fp8_quantize_dual", c10::DispatchKey::CUDA, TORCH_FN(driss_torch::mx_fp8_quantize_dual));
   m.def("mx_fp4_quantize(Tensor input, bool blocked, int axis) -> (Tensor, Tensor)");
   m.impl("mx_fp4_quantize", c10::DispatchKey::CUDA, TORCH_FN(driss_torch::mx_fp4_quantize));
+  m.def("mx_fp4_quantize_dual(Tensor input, bool blocked) -> (Tensor, Tensor, Tensor, Tensor)");
+  m.impl("mx_fp4_quantize_dual", c10::DispatchKey::CUDA, TORCH_FN(driss_torch::mx_fp4_quantize_dual));
   m.def("to_blocked(Tensor scale) -> Tensor");
   m.impl("to_blocked", c10::DispatchKey::CUDA, TORCH_FN(driss_torch::to_blocked));
 }

@@ -267,6 +267,18 @@ DT_API int dt_mx_fp4_bf16(const void* a, const void* b, const uint8_t* sfa, cons
 DT_API int dt_mx_fp4_quantize(const void* x, int in_dtype, int64_t rows, int64_t cols, int axis,
                               int scale_layout, void* data, uint8_t* scale, dt_stream_t stream);
 
+/* ------------------------------------------------------------- mx_fp4_quantize_dual --
+ * Both MXFP4 operands of x [rows, cols] from one read of it: the axis-1 cast (payload
+ * [rows, cols/2], scales [rows, cols/32]) and the axis-0 cast (payload [cols, rows/2], scales
+ * [cols, rows/32]), bit-identical to two calls of dt_mx_fp4_quantize.  No counterpart in the
+ * reference (see dt_mx_fp4_quantize); the MXFP4 sibling of dt_mx_fp8_quantize_dual.
+ * rows % 32 == 0 and cols % 32 == 0.  One kernel when data_rows is 4-byte, data_cols_t 16-byte and
+ * both scale buffers 4-byte aligned and rows, cols < 2^31; otherwise the two single casts with
+ * their own rules.                                                                            */
+DT_API int dt_mx_fp4_quantize_dual(const void* x, int in_dtype, int64_t rows, int64_t cols,
+                                   int scale_layout, void* data_rows, uint8_t* scale_rows,
+                                   void* data_cols_t, uint8_t* scale_cols_t, dt_stream_t stream);
+
 /* ------------------------------------------------- block-scaled GEMM with a workspace --
  * dt_mx_fp8_bf16 / dt_mx_fp4_bf16 (src/mx_fp8_bf16.cu:217-271; the reference takes its GEMM
  * workspace from the caching allocator at :148-151) with a caller-owned workspace of

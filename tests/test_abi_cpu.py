@@ -108,6 +108,13 @@ def test_host_validation_without_gpu():
     assert L.dt_mx_fp8_quantize_dual(fake, cabi.BF16, 128, 128, cabi.E4M3FN, 0, fake, fake, None, fake, None) == 3
     assert L.dt_mx_fp8_quantize_dual(fake + 1, cabi.BF16, 128, 128, cabi.E4M3FN, 0, fake, fake, fake, fake, None) == 4
     assert L.dt_mx_fp8_quantize_dual(None, cabi.BF16, 0, 128, cabi.E4M3FN, 0, None, None, None, None, None) == 0
+    assert L.dt_mx_fp4_quantize_dual(fake, cabi.BF16, 128, 48, 0, fake, fake, fake, fake, None) == 2
+    assert L.dt_mx_fp4_quantize_dual(fake, cabi.BF16, 48, 128, 0, fake, fake, fake, fake, None) == 2
+    assert L.dt_mx_fp4_quantize_dual(fake, cabi.BF16, 128, 128, 2, fake, fake, fake, fake, None) == 6
+    assert L.dt_mx_fp4_quantize_dual(fake, 9, 128, 128, 0, fake, fake, fake, fake, None) == 1
+    assert L.dt_mx_fp4_quantize_dual(fake, cabi.BF16, 128, 128, 0, fake, fake, None, fake, None) == 3
+    assert L.dt_mx_fp4_quantize_dual(fake + 1, cabi.BF16, 128, 128, 0, fake, fake, fake, fake, None) == 4
+    assert L.dt_mx_fp4_quantize_dual(None, cabi.BF16, 0, 128, 0, None, None, None, None, None) == 0
     assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 128, 128, 80, 80, 80, fake, 128, None) == 2  # K % 32
     assert L.dt_mx_fp8_bf16(fake, fake, fake, fake, 128, 126, 128, 128, 128, fake, 126, None) == 2  # N % 4
     assert L.dt_mx_fp8_bf16(fake + 8, fake, fake, fake, 128, 128, 128, 128, 128, fake, 128, None) == 4

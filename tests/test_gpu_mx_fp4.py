@@ -281,7 +281,7 @@ def _check_fp4_cast_cols(d, x):
 
 
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32, torch.float16])
-@pytest.mark.parametrize("shape", [(32, 128), (64, 4), (96, 76), (256, 512), (1024, 384), (160, 1028), (4096, 2048)],
+@pytest.mark.parametrize("shape", [(32, 128), (64, 4), (96, 76), (256, 512), (1024, 384), (160, 1028), (4096, 2048), (4128, 4104)],
                          ids=lambda s: f"{s[0]}x{s[1]}")
 def test_mx_fp4_cast_down_the_columns(d, in_dtype, shape):
     g = util.gen(shape[0] * 3 + shape[1])
@@ -289,6 +289,21 @@ def test_mx_fp4_cast_down_the_columns(d, in_dtype, shape):
     if in_dtype == torch.float16:
         x = x.clamp(-6.0e4, 6.0e4)
     _check_fp4_cast_cols(d, x.to(in_dtype))
+
+
+def test_mx_fp4_cast_down_the_columns_both_kernels(d, cabi):
+    """large 16-bit inputs take the one-read kernel without its row-wise half on a grid of walking
+    workgroups, everything else the kernel with 32-row lanes: the same bytes (8192 x 8192 and a ragged shape)"""
+    for shape in ((8192, 8192), (4128, 4360)):
+        x = util.normal(shape, 51, torch.bfloat16).cuda()
+        got = {}
+        for via in (1, 0):
+            cabi.set_tuning("mx.colt_via_dual", via)
+            try:
+                got[via] = d.mx_fp4_quantize(x, True, 0)
+            finally:
+                cabi.set_tuning("mx.colt_via_dual", 1)
+        assert torch.equal(got[0][0], got[1][0]) and torch.equal(util.codes(got[0][1]), util.codes(got[1][1]))
 
 
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
@@ -369,3 +384,106 @@ def test_mx_fp4_cast_errors_and_compile(d, cabi):
     fn = torch.compile(lambda t: d.mx_fp4_quantize(t, True), fullgraph=True, backend="aot_eager")
     got, want = fn(x), d.mx_fp4_quantize(x, True)
     assert torch.equal(got[0], want[0]) and torch.equal(util.codes(got[1]), util.codes(want[1]))
+
+
+# ------------------------------------------------- both MXFP4 operands from one read of x
+def _check_fp4_dual(d, x):
+    """mx_fp4_quantize_dual against the C oracle's cast of x (rows) and of x^T (columns, transposed)"""
+    M, N = x.shape
+    rd, rs = co.mx_fp4_quantize(x)
+    cd, cs = co.mx_fp4_quantize(x.t().contiguous())
+    for blocked in (False, True):
+        dr, sr, dc, sc = d.mx_fp4_quantize_dual(x.cuda(), blocked)
+        assert dr.dtype == torch.uint8 and dr.shape == (M, N // 2) and dc.shape == (N, M // 2)
+        assert sr.dtype == torch.float8_e8m0fnu and sc.dtype == torch.float8_e8m0fnu
+        assert torch.equal(dr.cpu(), rd) and torch.equal(dc.cpu(), cd)
+        assert torch.equal(util.codes(sr), (co.to_blocked(rs) if blocked else rs).flatten())
+        assert torch.equal(util.codes(sc), (co.to_blocked(cs) if blocked else cs).flatten())
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("shape", [(32, 32), (128, 256), (96, 160), (160, 96), (512, 1056), (1056, 512), (2048, 4096), (4128, 288)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+def test_mx_fp4_dual_against_oracle(d, in_dtype, shape):
+    """whole and ragged tiles (128 rows x 256 or 128 columns), wide-range data"""
+    g = util.gen(shape[0] * 5 + shape[1])
+    x = torch.randn(shape, generator=g) * torch.exp(2.0 * torch.randn(shape, generator=g))
+    if in_dtype == torch.float16:
+        x = x.clamp(-6.0e4, 6.0e4)
+    _check_fp4_dual(d, x.to(in_dtype))
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
+def test_mx_fp4_dual_special_blocks(d, in_dtype):
+    x = util.normal((128, 512), 45, in_dtype)
+    tiny = torch.finfo(in_dtype).tiny
+    x[0, :32] = 0.0
+    x[:32, 7] = 0.0
+    x[1, 32:64] = tiny / 4
+    x[2, 5] = float("inf")
+    x[3, 40] = float("-inf")
+    x[4, 70] = float("nan")
+    x[5, 100] = float("nan")
+    x[5, 101] = float("inf")
+    x[6, :32] = torch.finfo(in_dtype).max
+    x[64:96, 300] = torch.finfo(in_dtype).max
+    x[7, :32] = tiny
+    x[8, :32] = (torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0] * 4)).to(in_dtype)
+    x[96:128, 9] = -x[8, :32]
+    _check_fp4_dual(d, x)
+
+
+def test_mx_fp4_dual_matches_the_single_casts_at_full_size(d):
+    """8192 x 8192 bf16: the one-read kernel against the two single casts, both scale layouts"""
+    x = util.normal((8192, 8192), 46, torch.bfloat16).cuda()
+    for blocked in (False, True):
+        dr, sr, dc, sc = d.mx_fp4_quantize_dual(x, blocked)
+        wr, wsr = d.mx_fp4_quantize(x, blocked, 1)
+        wc, wsc = d.mx_fp4_quantize(x, blocked, 0)
+        assert torch.equal(dr, wr) and torch.equal(dc, wc)
+        assert torch.equal(util.codes(sr), util.codes(wsr)) and torch.equal(util.codes(sc), util.codes(wsc))
+
+
+def test_mx_fp4_dual_feeds_the_gemm_both_ways(d):
+    """x [M, K] cast once: its row operand in x @ w^T and its transposed operand in x^T @ g"""
+    M, K, N = 256, 512, 384
+    x, w, g = util.normal((M, K), 47), util.normal((N, K), 48), util.normal((N, M), 49)
+    xr, xrs, xt, xts = d.mx_fp4_quantize_dual(x.cuda(), True)
+    wd, ws = d.mx_fp4_quantize(w.cuda(), True)
+    gd, gs = d.mx_fp4_quantize(g.cuda(), True)
+    fwd = d.mx_fp4_bf16(xr, wd.t(), xrs, ws)                    # [M, N] = x w^T
+    wgrad = d.mx_fp4_bf16(xt, gd.t(), xts, gs)                  # [K, N] = x^T g^T
+    assert eager.compute_error(x.double() @ w.double().T, fwd.cpu().double()).item() > 15
+    assert eager.compute_error(x.double().T @ g.double().T, wgrad.cpu().double()).item() > 15
+
+
+def test_mx_fp4_dual_errors_fallback_and_compile(d, cabi):
+    x = util.normal((128, 256), 50).cuda()
+    with pytest.raises(RuntimeError):
+        d.mx_fp4_quantize_dual(x[:, :48].contiguous())   # 48 % 32
+    with pytest.raises(RuntimeError):
+        d.mx_fp4_quantize_dual(x[:48].contiguous())
+    with pytest.raises(RuntimeError):
+        d.mx_fp4_quantize_dual(x.t())                    # not contiguous
+    e = d.mx_fp4_quantize_dual(x[:0])
+    assert e[0].shape == (0, 128) and e[2].shape == (256, 0)
+    want = d.mx_fp4_quantize_dual(x, True)
+    cabi.set_tuning("mx.dual", 0)                        # the two single casts behind the same entry point
+    try:
+        two = d.mx_fp4_quantize_dual(x, True)
+    finally:
+        cabi.set_tuning("mx.dual", 1)
+    for a, b in zip(want, two):
+        assert torch.equal(util.codes(a), util.codes(b))
+    L = cabi.lib()
+    buf = torch.empty(4 * 128 * 256, dtype=torch.uint8, device="cuda")
+    p = buf.data_ptr()
+    assert L.dt_mx_fp4_quantize_dual(x.data_ptr(), cabi.BF16, 128, 48, 0, p, p, p, p, None) == 2
+    assert L.dt_mx_fp4_quantize_dual(x.data_ptr(), cabi.BF16, 128, 256, 2, p, p, p, p, None) == 6
+    assert L.dt_mx_fp4_quantize_dual(x.data_ptr(), 9, 128, 256, 0, p, p, p, p, None) == 1
+    assert L.dt_mx_fp4_quantize_dual(x.data_ptr(), cabi.BF16, 128, 256, 0, p, p, None, p, None) == 3
+    assert L.dt_mx_fp4_quantize_dual(None, cabi.BF16, 0, 256, 0, None, None, None, None, None) == 0
+    fn = torch.compile(lambda t: d.mx_fp4_quantize_dual(t, True), fullgraph=True, backend="aot_eager")
+    got = fn(x)
+    for a, b in zip(got, want):
+        assert torch.equal(util.codes(a), util.codes(b))
