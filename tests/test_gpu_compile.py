@@ -131,7 +131,7 @@ def test_ops_replay_from_a_captured_graph(d):
         return (d.mx_fp8_bf16(a2, b2.t(), sa2, sb2), d.amax(x), d.saturated_cast(x, scale, E4), d.dynamic_scaled_quant(x, E5),
                 d.dynamic_scaled_quant_pair(x), d.dynamic_scaled_quant_rowwise(x, E4), d.mx_fp8_quantize(x),
                 d.mx_fp8_quantize(x, 32, 0, True), d.mx_fp8_quantize_dual(x, E4, True), d.mx_fp8_bf16(a, b.t(), sa, sb),
-                d.mx_fp4_quantize(x, True))
+                d.mx_fp4_quantize(x, True), d.mx_fp4_quantize_dual(x, True))
 
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
